@@ -1,0 +1,147 @@
+"""Pins the oracle's number formats against library routines that are independent of it (numpy float16,
+torch bfloat16 / float8_e4m3fn) and against closed forms.  CPU only."""
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+GOLD = Path(__file__).parent / "golden"
+
+
+def test_f16_decode_all_codes(oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    ref = bits.view(np.float16).astype(np.float32)
+    got = np.array([oracle.lib.orc_f16_to_f32(int(b)) for b in bits], np.float32)
+    both_nan = np.isnan(ref) & np.isnan(got)
+    assert np.array_equal(ref.view(np.uint32)[~both_nan], got.view(np.uint32)[~both_nan])
+
+
+def test_f16_encode_rne(oracle):
+    rng = np.random.default_rng(0)
+    x = np.concatenate([
+        rng.standard_normal(20000) * 10.0 ** rng.uniform(-8, 5, 20000),
+        # exact ties between neighbouring halfs and values one ulp(f64) either side
+        (np.arange(1, 2047, dtype=np.float64) + 0.5) * 2.0 ** -14, (np.arange(1, 2047) + 0.5) * 2.0 ** -24 * 1024,
+        np.nextafter((np.arange(1, 2047, dtype=np.float64) + 0.5) * 2.0 ** -3, 0), np.nextafter((np.arange(1, 2047, dtype=np.float64) + 0.5) * 2.0 ** -3, 9e9),
+        [0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e6, -1e6, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0000001, 5.96e-8, 6.1e-5],
+    ])
+    ref = x.astype(np.float16).view(np.uint16)           # numpy converts binary64 -> binary16 with one rounding
+    got = np.array([oracle.lib.orc_f64_to_f16(float(v)) for v in x], np.uint16)
+    assert np.array_equal(ref, got)
+
+
+def test_bf16_rne_vs_torch(oracle):
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal(50000) * 10.0 ** rng.uniform(-6, 6, 50000)).astype(np.float32)
+    ties = (np.arange(0x3f80, 0x4080, dtype=np.uint32) << 16 | 0x8000).view(np.float32)   # exact ties
+    x = np.concatenate([x, ties, np.nextafter(ties, 0), np.nextafter(ties, np.float32(9e9))]).astype(np.float32)
+    ref = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = np.array([oracle.lib.orc_f32_to_bf16(float(v)) for v in x], np.uint16)
+    assert np.array_equal(ref, got)
+    assert np.array_equal(oracle.bf16_bits(x), ref)      # the numpy helper used by the generators
+
+
+def test_e4m3_decode_all_codes_vs_torch(oracle):
+    codes = torch.arange(256, dtype=torch.uint8)
+    ref = codes.view(torch.float8_e4m3fn).float().numpy()
+    got = np.array([oracle.lib.orc_e4m3_to_f32(int(c)) for c in range(256)], np.float32)
+    nan = np.isnan(ref)
+    assert np.array_equal(nan, np.isnan(got)) and nan.sum() == 2
+    assert np.array_equal(ref[~nan], got[~nan])
+    assert got[0x7e] == 448.0 and got[0x08] == 2.0 ** -6 and got[0x01] == 2.0 ** -9      # OCP FP8 anchors
+
+
+def test_e4m3_encode_rne_vs_torch(oracle):
+    rng = np.random.default_rng(2)
+    vals = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    vals = np.sort(vals[np.isfinite(vals)])
+    mids = (vals[:-1].astype(np.float64) + vals[1:]) / 2                  # exact ties (representable in binary32)
+    x = np.concatenate([vals, mids, np.nextafter(mids.astype(np.float32), -9e9), np.nextafter(mids.astype(np.float32), 9e9),
+                        rng.uniform(-448, 448, 40000), rng.standard_normal(20000) * 10.0 ** rng.uniform(-5, 0, 20000)]).astype(np.float32)
+    x = x[np.abs(x) <= 448.0]
+    ref = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = np.array([oracle.lib.orc_f32_to_e4m3(float(v)) for v in x], np.uint8)
+    # +0 and -0 both decode to zero; compare the codes exactly except the sign of zero
+    z = (ref & 0x7f) == 0
+    assert np.array_equal(ref[~z], got[~z]) and np.all((got[z] & 0x7f) == 0)
+    # saturation: beyond the largest finite value the conversion gives +-448 (the clamp of the reference kernels)
+    assert oracle.lib.orc_f32_to_e4m3(1e9) == 0x7e and oracle.lib.orc_f32_to_e4m3(-500.0) == 0xfe
+
+
+def test_e8m0_and_e2m1(oracle):
+    for b in range(1, 255):
+        assert oracle.lib.orc_e8m0_to_f32(b) == 2.0 ** (b - 127)
+    assert oracle.lib.orc_e8m0_to_f32(0) == 0.0            # reference ops.rs:22 / ds41.cu:23: the bits b << 23
+    table = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]       # OCP MX E2M1 magnitudes
+    for c in range(16):
+        v = oracle.lib.orc_e2m1_to_f32(c)
+        assert abs(v) == table[c & 7] and (np.signbit(v) == bool(c & 8))
+
+
+def test_mxfp4_dequant_exhaustive(oracle):
+    # every byte (two codes) x every usable scale byte, against the closed form table[nibble] * 2^(s - 127)
+    table = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0., -.5, -1, -1.5, -2, -3, -4, -6], np.float64)
+    scales = np.arange(1, 253, dtype=np.uint8)                 # 6 * 2^(253-127) would overflow binary32
+    w = np.tile(np.arange(256, dtype=np.uint8).reshape(16, 16), (len(scales), 1))        # [252*16, 16] -> K = 32
+    s = np.repeat(scales, 16).reshape(-1, 1)
+    got = oracle.mxfp4_dequant(w, s)
+    lo, hi = w & 15, w >> 4
+    ref = np.stack([table[lo], table[hi]], -1).reshape(w.shape[0], 32) * 2.0 ** (s.astype(np.float64) - 127)
+    assert np.array_equal(got.astype(np.float64), ref)     # low nibble = even k
+
+
+def test_fp8_block_dequant_closed_form(oracle):
+    rng = np.random.default_rng(3)
+    w = rng.integers(0, 256, (256, 384), dtype=np.uint8)
+    w[(w & 0x7f) == 0x7f] = 0
+    s = np.exp(rng.uniform(np.log(1e-3), np.log(1e-1), (2, 3))).astype(np.float32)
+    got = oracle.fp8_block_dequant(w, s, 128)
+    ref = torch.from_numpy(w).view(torch.float8_e4m3fn).float().numpy() * np.repeat(np.repeat(s, 128, 0), 128, 1)
+    assert np.array_equal(got, ref.astype(np.float32))
+    s8 = rng.integers(100, 130, (8, 12), dtype=np.uint8)
+    got = oracle.fp8_e8m0_dequant(w, s8)
+    ref = torch.from_numpy(w).view(torch.float8_e4m3fn).float().numpy() * np.repeat(np.repeat(2.0 ** (s8.astype(np.float32) - 127), 32, 0), 32, 1)
+    assert np.array_equal(got, ref.astype(np.float32))
+
+
+def _act_quant_torch(x):
+    """act_quant with UE8M0 scales per 32 from library pieces only (torch float8 cast, frexp): the closed form
+    scale = 2^ceil(log2(max(amax, 1e-4) / 448)), q = e4m3_rn(clamp(x / scale))."""
+    xb = x.float().reshape(-1, 32)
+    amax = xb.abs().amax(-1).clamp_min(1e-4)
+    t = amax * torch.tensor(1.0 / 448.0)
+    m, e = torch.frexp(t)                                   # t = m * 2^e, m in [0.5, 1)
+    ce = torch.where(m == 0.5, e - 1, e)                    # ceil(log2 t)
+    s = torch.ldexp(torch.ones_like(t), ce)
+    q = (xb / s[:, None]).clamp(-448, 448).to(torch.float8_e4m3fn)
+    return q.view(torch.uint8).reshape(x.shape).numpy(), (ce + 127).to(torch.uint8).reshape(*x.shape[:-1], -1).numpy(), \
+        (q.float() * s[:, None]).reshape(x.shape).to(torch.bfloat16)
+
+
+def test_act_quant_vs_library(oracle):
+    g = torch.Generator().manual_seed(4)
+    # blocks whose amax sweeps many binades (incl. below the 1e-4 floor and exact powers of two times 448)
+    x = torch.randn(4096, 32, generator=g) * (10.0 ** torch.empty(4096, 1).uniform_(-6, 3, generator=g))
+    x[:64] = 0.0
+    x[64:128, 0] = 448.0 * 2.0 ** torch.arange(-32, 32).float()[:64]
+    x = x.to(torch.bfloat16)
+    q_ref, s_ref, d_ref = _act_quant_torch(x)
+    bits = x.view(torch.int16).numpy().view(np.uint16)
+    q, s = oracle.act_quant_fp8(bits)
+    assert np.array_equal(s, s_ref)
+    z = (q_ref & 0x7f) == 0
+    assert np.array_equal(q[~z], q_ref[~z]) and np.all((q[z] & 0x7f) == 0)
+    d = oracle.act_quant32(bits)
+    assert np.array_equal(oracle.bf16_to_f32(d), d_ref.float().numpy())
+
+
+def test_act_quant_scale_exhaustive_exponents(oracle):
+    # aq_scale over every binade and mantissa pattern class: exact power of two vs not
+    for e in range(-20, 12):
+        for man in (1.0, 1.0 + 2.0 ** -23, 1.5, 2.0 - 2.0 ** -23):
+            amax = np.float32(man * 2.0 ** e)
+            t = np.float32(max(amax, np.float32(1e-4))) * np.float32(1.0 / 448.0)
+            expect = int(np.ceil(np.log2(np.float64(t)))) + 127
+            assert oracle.lib.orc_aq_scale(float(amax)) == expect, (e, man)
