@@ -1,0 +1,114 @@
+// Shared device helpers for the gfx950 (CDNA4, wave64) kernels of the quantized MoE expert path.
+// Everything here is written for one target: no other architecture is supported.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define SPARK_API extern "C" __attribute__((visibility("default")))
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+namespace spk {
+
+constexpr int WAVE = 64;
+
+// ---- number formats (bit-exact, software: the bytes must match the CPU reference of the same rule) ----
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7f800000u) == 0x7f800000u && (u & 0x7fffffu)) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float bf16_round(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { _Float16 v; __builtin_memcpy(&v, &h, 2); return (float)v; }
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { _Float16 v = (_Float16)f; uint16_t h; __builtin_memcpy(&h, &v, 2); return h; }   // RNE
+// E8M0 scale byte -> 2^(b-127) from the exponent bits (byte 0 gives 0.0)
+__device__ __forceinline__ float e8m0_to_f32(uint32_t b) { return __uint_as_float(b << 23); }
+// OCP E4M3 (fn) -> binary32.  Exponent and mantissa are dropped into binary32 and rescaled by 2^120, which also maps the
+// subnormal codes exactly; done with integer arithmetic so that it does not depend on the denormal mode.
+__device__ __forceinline__ float e4m3_to_f32(uint32_t b)
+{
+    const uint32_t s = (b & 0x80u) << 24, em = b & 0x7fu;
+    if ((em >> 3) == 0) return __uint_as_float(s | __float_as_uint((float)(em & 7u) * 0.001953125f));
+    return __uint_as_float(s | ((em << 20) + (120u << 23)));
+}
+// binary32 (already clamped to [-448, 448]) -> E4M3 code, round to nearest even
+__device__ __forceinline__ uint32_t f32_to_e4m3(float f)
+{
+    const uint32_t u = __float_as_uint(f), s = (u >> 24) & 0x80u, a = u & 0x7fffffffu;
+    const float af = __uint_as_float(a);
+    if (af >= 448.0f) return s | 0x7eu;
+    const int e = (int)(a >> 23) - 127;
+    if (e < -6) return s | (uint32_t)__builtin_rintf(af * 512.0f);   // units of 2^-9, ties to even; 8 = smallest normal
+    const uint32_t m = a & 0x7fffffu;
+    uint32_t q = m >> 20;
+    const uint32_t rem = m & 0xfffffu;
+    q += (rem > 0x80000u || (rem == 0x80000u && (q & 1u))) ? 1u : 0u;
+    uint32_t r = ((uint32_t)(e + 7) << 3) + q;
+    return s | (r > 0x7eu ? 0x7eu : r);
+}
+// act_quant: UE8M0 scale byte of a 32-block from its absolute maximum, and the E4M3 byte of one value under it
+__device__ __forceinline__ uint32_t aq_scale(float amax)
+{
+    amax = fmaxf(amax, 1e-4f);
+    const uint32_t bits = __float_as_uint(amax * (1.0f / 448.0f));
+    return ((bits >> 23) & 0xffu) + ((bits & 0x7fffffu) != 0u ? 1u : 0u);
+}
+__device__ __forceinline__ uint32_t aq_byte(float v, uint32_t e)
+{
+    const float s = __uint_as_float(e << 23);
+    return f32_to_e4m3(fminf(fmaxf(v / s, -448.f), 448.f));
+}
+__device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
+
+// ---- wave64 cross-lane primitives ----
+// value of lane (lane ^ mask) for mask < 64
+__device__ __forceinline__ float xor_f(float v, int mask) { return __shfl_xor(v, mask, 64); }
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// 128-point normalized Walsh-Hadamard over values held 2 per lane (lane l: elements 2l, 2l+1), binary32, butterflies
+// h = 1, 2, ..., 64 with (a + b, a - b), lower index first, then one multiply: the operation order of a serial FWHT.
+__device__ __forceinline__ void fwht128(float& v0, float& v1, int lane)
+{
+    { const float a = v0 + v1, b = v0 - v1; v0 = a; v1 = b; }
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) {
+        const bool upper = lane & m;
+        const float o0 = __shfl_xor(v0, m, 64), o1 = __shfl_xor(v1, m, 64);
+        v0 = upper ? o0 - v0 : v0 + o0;
+        v1 = upper ? o1 - v1 : v1 + o1;
+    }
+    v0 *= 0.08838834764831845f;
+    v1 *= 0.08838834764831845f;
+}
+
+// 16-byte streaming load (weights are read once: keep them out of the way of reused data)
+__device__ __forceinline__ uint4 ld_stream16(const void* p)
+{
+    typedef const __attribute__((address_space(1))) v4i* gptr;   // global memory: a plain global_load, never a flat one
+    const v4i v = __builtin_nontemporal_load((gptr)(uintptr_t)p);
+    return make_uint4((uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w);
+}
+
+inline int launch_status() { return (int)hipGetLastError(); }
+inline size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+}  // namespace spk

@@ -1,0 +1,76 @@
+// EXL3 trellis decode primitives for wave64.
+//
+// Format (reference engine-rs/shim/qwen_exl3.cuh:8-11, reference/qwen38/exl3.py:1-15): a 16x16 weight tile is 16*bits
+// int16 words = 8*bits little-endian uint32, read MSB-first as one tail-biting bitstream of 256*bits bits.  The 16-bit
+// state of sequence position p starts at bit ((p+1)*bits - 16) mod (256*bits).  Position 8t+j is tile element
+// row (t%4)*2 + {0,1,8,9}[j%4], column t/4 + 8*(j/4).  A codebook maps the state to an fp16 value.
+#pragma once
+#include "common.hpp"
+
+namespace spk {
+
+// codebook ids follow the reference (moe_exl3.cuh:6): 2 = mul1 (Qwen), 1 = mcg (GLM)
+constexpr int CB_MCG = 1, CB_MUL1 = 2;
+
+// reference qwen_exl3.cuh:17-23: x = state * 0x83DCD12D, b = sum of the 4 bytes, fp16 fma(1024 + b, 0x1eee, 0xc931)
+__device__ __forceinline__ _Float16 mul1_decode(uint32_t state)
+{
+    const uint32_t x = state * 0x83DCD12Du;
+    const uint32_t s = __builtin_amdgcn_sad_u8(x, 0u, 0x6400u);          // 0x6400 + byte sum = fp16 bits of 1024 + b
+    _Float16 h, c1, c2;
+    const uint16_t hs = (uint16_t)s, k1 = 0x1eee, k2 = 0xc931;
+    __builtin_memcpy(&h, &hs, 2); __builtin_memcpy(&c1, &k1, 2); __builtin_memcpy(&c2, &k2, 2);
+    return __builtin_fmaf16(h, c1, c2);                                  // one rounding
+}
+// reference qwen_exl3.cuh:26-32: x = state * 0xCBAC1FED, (x & 0x8fff8fff) ^ 0x3b603b60 as two fp16, added in fp16
+__device__ __forceinline__ _Float16 mcg_decode(uint32_t state)
+{
+    uint32_t x = state * 0xCBAC1FEDu;
+    x = (x & 0x8fff8fffu) ^ 0x3b603b60u;
+    h2 v; __builtin_memcpy(&v, &x, 4);
+    return v.x + v.y;
+}
+template <int CBK> __device__ __forceinline__ _Float16 cb_decode(uint32_t state)
+{
+    return CBK == CB_MCG ? mcg_decode(state) : mul1_decode(state);
+}
+// Two states -> packed fp16 pair (low half = state a): the same fp16 operation per element as cb_decode.
+template <int CBK> __device__ __forceinline__ h2 cb_decode2(uint32_t a, uint32_t b)
+{
+    if constexpr (CBK == CB_MCG) {
+        uint32_t x0 = a * 0xCBAC1FEDu, x1 = b * 0xCBAC1FEDu;
+        x0 = (x0 & 0x8fff8fffu) ^ 0x3b603b60u;
+        x1 = (x1 & 0x8fff8fffu) ^ 0x3b603b60u;
+        const uint32_t lo = __builtin_amdgcn_perm(x1, x0, 0x05040100u);   // (x0.lo16, x1.lo16)
+        const uint32_t hi = __builtin_amdgcn_perm(x1, x0, 0x07060302u);   // (x0.hi16, x1.hi16)
+        h2 l, h; __builtin_memcpy(&l, &lo, 4); __builtin_memcpy(&h, &hi, 4);
+        return l + h;
+    } else {
+        uint32_t s = __builtin_amdgcn_sad_u8(a * 0x83DCD12Du, 0u, 0x64006400u);
+        s = __builtin_amdgcn_sad_hi_u8(b * 0x83DCD12Du, 0u, s);          // (0x6400 + sum a) | (0x6400 + sum b) << 16
+        h2 h; __builtin_memcpy(&h, &s, 4);
+        const uint32_t k1 = 0x1eee1eeeu, k2 = 0xc931c931u;
+        h2 c1, c2; __builtin_memcpy(&c1, &k1, 4); __builtin_memcpy(&c2, &k2, 4);
+        return __builtin_elementwise_fma(h, c1, c2);
+    }
+}
+
+// State of sequence position p of a tile of `bits` bits per weight; w = the tile's 8*bits uint32 words (any memory).
+__device__ __forceinline__ uint32_t tile_state(const uint32_t* w, int bits, int p)
+{
+    const int nw = 8 * bits, L = 256 * bits;
+    int b0 = ((p + 1) * bits - 16) % L;
+    if (b0 < 0) b0 += L;
+    const int i0 = b0 >> 5, i1 = (i0 + 1 == nw) ? 0 : i0 + 1;
+    const uint64_t win = ((uint64_t)w[i0] << 32) | w[i1];
+    return (uint32_t)(win >> (48 - (b0 & 31))) & 0xffffu;
+}
+// tile element (row, col) of sequence position p
+__device__ __forceinline__ void tile_pos(int p, int& row, int& col)
+{
+    const int t = p >> 3, j = p & 7;
+    row = (t & 3) * 2 + (j & 1) + ((j & 2) ? 8 : 0);
+    col = (t >> 2) + ((j & 4) ? 8 : 0);
+}
+
+}  // namespace spk

@@ -1,0 +1,259 @@
+// Dequantisation surfaces (bit-exact against the reference's dequant) and activation quantisation.
+//   EXL3 reconstruct / fold      reference engine-rs/shim/qwen_exl3.cuh:629-701, qwen_exl3.cu (entry points)
+//   MXFP4 / FP8 block dequant    reference reference/ds41/kernel.py:96-99,122-131
+//   act_quant (UE8M0 per 32)     reference engine-rs/shim/ds41.cu:148-164, ds41_mx.cu:42-51,320-331
+//   shared-expert glue           reference engine-rs/shim/ds41_ops.cu:421-442, qwen_moe.cu:69-84
+#include "common.hpp"
+#include "exl3_decode.hpp"
+
+using namespace spk;
+
+namespace {
+
+// ---------------------------------------------------------------- EXL3 reconstruct: one workgroup of 256 per tile
+template <int CBK>
+__global__ __launch_bounds__(256) void exl3_reconstruct_kernel(const uint32_t* __restrict__ tr, uint16_t* __restrict__ w, int K, int N, int bits)
+{
+    __shared__ uint32_t tw[48];
+    const int nw = 8 * bits, Nt = N / 16;
+    const int64_t tile = blockIdx.x;
+    const int kt = (int)(tile / Nt), nt = (int)(tile % Nt), p = threadIdx.x;
+    if (p < nw) tw[p] = tr[tile * nw + p];
+    __syncthreads();
+    int row, col;
+    tile_pos(p, row, col);
+    const _Float16 v = cb_decode<CBK>(tile_state(tw, bits, p));
+    uint16_t hb; __builtin_memcpy(&hb, &v, 2);
+    w[(int64_t)(kt * 16 + row) * N + nt * 16 + col] = hb;
+}
+
+// ---------------------------------------------------------------- EXL3 fold: W^T [N, K] fp16 = (diag(suh) H inner H diag(svh))^T
+// One 128 x 128 block per workgroup of 256 threads: decode into LDS (k-major), Hadamard along k then * suh[k],
+// Hadamard along n then * svh[n], all binary32 in the operation order of the reference kernel (bit-identical results).
+constexpr int FOLD_LD = 129;
+template <int CBK>
+__global__ __launch_bounds__(256) void exl3_fold_kernel(const uint32_t* __restrict__ tr, const uint16_t* __restrict__ suh, const uint16_t* __restrict__ svh,
+                                                        int K, int N, int bits, uint16_t* __restrict__ out, int64_t ldo)
+{
+    extern __shared__ float fs[];                    // [128][FOLD_LD] k-major, then 64 tiles' words
+    uint32_t* tw = (uint32_t*)(fs + 128 * FOLD_LD);  // [64][48]
+    const int nb = blockIdx.x, kb = blockIdx.y, Nt = N / 16, nw = 8 * bits;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    for (int i = tid; i < 64 * nw; i += 256) {
+        const int t = i / nw, j = i % nw;
+        const int kt = kb * 8 + t / 8, nt = nb * 8 + t % 8;
+        tw[t * 48 + j] = tr[((int64_t)kt * Nt + nt) * nw + j];
+    }
+    __syncthreads();
+    {
+        int row, col;
+        tile_pos(tid, row, col);
+        for (int t = 0; t < 64; ++t) {
+            const _Float16 v = cb_decode<CBK>(tile_state(tw + t * 48, bits, tid));
+            fs[((t / 8) * 16 + row) * FOLD_LD + (t % 8) * 16 + col] = (float)v;
+        }
+    }
+    __syncthreads();
+    for (int c = wave; c < 128; c += 4) {            // H along k, then * suh[k]
+        float v0 = fs[(2 * lane) * FOLD_LD + c], v1 = fs[(2 * lane + 1) * FOLD_LD + c];
+        fwht128(v0, v1, lane);
+        fs[(2 * lane) * FOLD_LD + c] = v0 * f16_bits_to_f32(suh[kb * 128 + 2 * lane]);
+        fs[(2 * lane + 1) * FOLD_LD + c] = v1 * f16_bits_to_f32(suh[kb * 128 + 2 * lane + 1]);
+    }
+    __syncthreads();
+    for (int r = wave; r < 128; r += 4) {            // H along n, then * svh[n]
+        float v0 = fs[r * FOLD_LD + 2 * lane], v1 = fs[r * FOLD_LD + 2 * lane + 1];
+        fwht128(v0, v1, lane);
+        fs[r * FOLD_LD + 2 * lane] = v0 * f16_bits_to_f32(svh[nb * 128 + 2 * lane]);
+        fs[r * FOLD_LD + 2 * lane + 1] = v1 * f16_bits_to_f32(svh[nb * 128 + 2 * lane + 1]);
+    }
+    __syncthreads();
+    for (int i = tid; i < 128 * 128; i += 256) {
+        const int n = i / 128, k = i % 128;
+        out[(int64_t)(nb * 128 + n) * ldo + kb * 128 + k] = f32_to_f16_bits(fs[k * FOLD_LD + n]);
+    }
+}
+
+// ---------------------------------------------------------------- MXFP4 / FP8 dequant to binary32
+__global__ void mxfp4_dequant_kernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ s, float* __restrict__ out, int64_t nbytes, int K)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // packed byte index
+    if (i >= nbytes) return;
+    const int kb = K / 2;
+    const int64_t n = i / kb;
+    const int k = (int)(i % kb) * 2;
+    const uint32_t b = w[i];
+    const float sc = e8m0_to_f32(s[n * (K / 32) + k / 32]);
+    const v2f v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(b, 1.0f, 0);   // exact E2M1 -> binary32, low nibble first
+    out[n * K + k] = v.x * sc;
+    out[n * K + k + 1] = v.y * sc;
+}
+__global__ void fp8_block_dequant_kernel(const uint8_t* __restrict__ w, const float* __restrict__ s, float* __restrict__ out, int N, int K, int bs)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)N * K) return;
+    const int n = (int)(i / K), k = (int)(i % K), kbn = (K + bs - 1) / bs;
+    out[i] = e4m3_to_f32(w[i]) * s[(int64_t)(n / bs) * kbn + k / bs];
+}
+__global__ void fp8_e8m0_dequant_kernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ s, float* __restrict__ out, int N, int K)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)N * K) return;
+    const int n = (int)(i / K), k = (int)(i % K);
+    out[i] = e4m3_to_f32(w[i]) * e8m0_to_f32(s[(int64_t)(n >> 5) * (K >> 5) + (k >> 5)]);
+}
+
+// ---------------------------------------------------------------- act_quant: 32 lanes per block of 32, two blocks per wave
+template <bool BYTES>
+__global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ outb, uint8_t* __restrict__ q,
+                                                        uint8_t* __restrict__ s, int64_t blocks)
+{
+    const int64_t b = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
+    const int l = threadIdx.x & 31;
+    if (b >= blocks) return;
+    const float v = bf16_to_f32(x[b * 32 + l]);
+    float a = fabsf(v);
+#pragma unroll
+    for (int o = 16; o; o >>= 1) a = fmaxf(a, __shfl_xor(a, o, 64));     // stays inside the half-wave
+    const uint32_t e = aq_scale(a);
+    const uint32_t byte = aq_byte(v, e);
+    if (BYTES) {
+        q[b * 32 + l] = (uint8_t)byte;
+        if (l == 0) s[b] = (uint8_t)e;
+    } else {
+        outb[b * 32 + l] = f32_to_bf16(e4m3_to_f32(byte) * __uint_as_float(e << 23));
+    }
+}
+
+// gu [T, 2I] binary32 -> bf16 act-quantized silu(gate) * up; reference ds41_ops.cu:421-442
+__global__ __launch_bounds__(256) void swiglu_quant_kernel(const float* __restrict__ gu, uint16_t* __restrict__ out, int T, int I, float lim)
+{
+    const int64_t blk = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
+    const int l = threadIdx.x & 31;
+    if (blk >= (int64_t)T * (I / 32)) return;
+    const int row = (int)(blk / (I / 32)), j = (int)(blk % (I / 32)) * 32 + l;
+    float g = bf16_round(gu[(int64_t)row * 2 * I + j]);
+    float u = bf16_round(gu[(int64_t)row * 2 * I + I + j]);
+    if (lim > 0.f) { g = fminf(g, lim); u = fminf(fmaxf(u, -lim), lim); }
+    const float v = bf16_round(silu(g) * u);
+    float a = fabsf(v);
+#pragma unroll
+    for (int o = 16; o; o >>= 1) a = fmaxf(a, __shfl_xor(a, o, 64));
+    const uint32_t e = aq_scale(a);
+    out[(int64_t)row * I + j] = f32_to_bf16(e4m3_to_f32(aq_byte(v, e)) * __uint_as_float(e << 23));
+}
+__global__ void silu_mul_kernel(const float* __restrict__ g, const float* __restrict__ u, float* __restrict__ h, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) h[i] = silu(g[i]) * u[i];
+}
+__global__ void gate_scale_kernel(const float* __restrict__ gl, int64_t ldg, int col, const float* __restrict__ d, float* __restrict__ out, int R, int N)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= R * N) return;
+    const float a = gl[(int64_t)(i / N) * ldg + col];
+    out[i] = (1.0f / (1.0f + expf(-a))) * d[i];
+}
+
+}  // namespace
+
+// ================================================================ C ABI
+
+// reference qwen_exl3.cu (qwen_exl3_reconstruct): trellis [K/16, N/16, 16*bits] int16 -> inner [K, N] fp16, mul1 codebook
+SPARK_API int spark_exl3_reconstruct(const void* trellis, void* w_f16, int K, int N, int bits, int codebook, hipStream_t st)
+{
+    if (K < 16 || N < 16 || K % 16 || N % 16 || bits < 3 || bits > 6) return -1;
+    if (codebook != CB_MCG && codebook != CB_MUL1) return -2;
+    const unsigned tiles = (unsigned)((K / 16) * (N / 16));
+    if (codebook == CB_MCG) exl3_reconstruct_kernel<CB_MCG><<<tiles, 256, 0, st>>>((const uint32_t*)trellis, (uint16_t*)w_f16, K, N, bits);
+    else exl3_reconstruct_kernel<CB_MUL1><<<tiles, 256, 0, st>>>((const uint32_t*)trellis, (uint16_t*)w_f16, K, N, bits);
+    return launch_status();
+}
+SPARK_API int qwen_exl3_reconstruct(const void* trellis, void* w_f16, int K, int N, int bits, hipStream_t st)
+{
+    return spark_exl3_reconstruct(trellis, w_f16, K, N, bits, CB_MUL1, st);
+}
+// reference qwen_exl3.cu (qwen_exl3_fold): out = W^T [N, K] fp16, row stride ldo
+SPARK_API int spark_exl3_fold(const void* trellis, const void* suh, const void* svh, int K, int N, int bits, int codebook, void* out_f16,
+                              int64_t ldo, hipStream_t st)
+{
+    if (K < 128 || N < 128 || K % 128 || N % 128 || bits < 3 || bits > 6 || ldo < K) return -1;
+    if (codebook != CB_MCG && codebook != CB_MUL1) return -2;
+    const size_t sm = 128 * FOLD_LD * 4 + 64 * 48 * 4;
+    static bool attr = hipFuncSetAttribute((const void*)exl3_fold_kernel<CB_MCG>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm) == hipSuccess &&
+                       hipFuncSetAttribute((const void*)exl3_fold_kernel<CB_MUL1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm) == hipSuccess;
+    if (!attr) return -3;
+    const dim3 grid(N / 128, K / 128);
+    if (codebook == CB_MCG) exl3_fold_kernel<CB_MCG><<<grid, 256, sm, st>>>((const uint32_t*)trellis, (const uint16_t*)suh, (const uint16_t*)svh, K, N, bits, (uint16_t*)out_f16, ldo);
+    else exl3_fold_kernel<CB_MUL1><<<grid, 256, sm, st>>>((const uint32_t*)trellis, (const uint16_t*)suh, (const uint16_t*)svh, K, N, bits, (uint16_t*)out_f16, ldo);
+    return launch_status();
+}
+SPARK_API int qwen_exl3_fold(const void* trellis, const void* suh, const void* svh, int K, int N, int bits, void* out_f16, int64_t ldo, hipStream_t st)
+{
+    return spark_exl3_fold(trellis, suh, svh, K, N, bits, CB_MUL1, out_f16, ldo, st);
+}
+
+// W [N, K/2] E2M1 pairs + S [N, K/32] E8M0 -> binary32 [N, K]
+SPARK_API int spark_mxfp4_dequant(const void* w, const void* s, float* out, int N, int K, hipStream_t st)
+{
+    if (N < 1 || K < 32 || K % 32) return 1;
+    const int64_t nbytes = (int64_t)N * K / 2;
+    mxfp4_dequant_kernel<<<(unsigned)((nbytes + 255) / 256), 256, 0, st>>>((const uint8_t*)w, (const uint8_t*)s, out, nbytes, K);
+    return launch_status();
+}
+// W [N, K] E4M3 + binary32 scale per bs x bs block -> binary32 [N, K]
+SPARK_API int spark_fp8_block_dequant(const void* w, const float* s, float* out, int N, int K, int bs, hipStream_t st)
+{
+    if (N < 1 || K < 1 || bs < 1) return 1;
+    const int64_t n = (int64_t)N * K;
+    fp8_block_dequant_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((const uint8_t*)w, s, out, N, K, bs);
+    return launch_status();
+}
+// W [N, K] E4M3 + E8M0 scale per 32 x 32 block -> binary32 [N, K]
+SPARK_API int spark_fp8_e8m0_dequant(const void* w, const void* s, float* out, int N, int K, hipStream_t st)
+{
+    if (N < 1 || K < 32 || K % 32) return 1;
+    const int64_t n = (int64_t)N * K;
+    fp8_e8m0_dequant_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((const uint8_t*)w, (const uint8_t*)s, out, N, K);
+    return launch_status();
+}
+
+// reference ds41.cu:274-278
+SPARK_API int ds41_act_quant32(const void* x, void* out, long long numel, hipStream_t st)
+{
+    if (numel % 32) return 1;
+    const long long blocks = numel / 32;
+    if (blocks == 0) return 0;
+    act_quant_kernel<false><<<(unsigned)((blocks + 7) / 8), 256, 0, st>>>((const uint16_t*)x, (uint16_t*)out, nullptr, nullptr, blocks);
+    return launch_status();
+}
+// reference ds41_mx.cu:1394-1399
+SPARK_API int ds41_act_quant_fp8(const void* x, void* q, void* s, long long numel, hipStream_t st)
+{
+    if (numel % 32) return 1;
+    const long long blocks = numel / 32;
+    if (blocks == 0) return 0;
+    act_quant_kernel<true><<<(unsigned)((blocks + 7) / 8), 256, 0, st>>>((const uint16_t*)x, nullptr, (uint8_t*)q, (uint8_t*)s, blocks);
+    return launch_status();
+}
+// reference ds41_ops.cu:615 (ds41_swiglu_quant)
+SPARK_API int ds41_swiglu_quant(const float* gu, void* out, int T, int I, float lim, hipStream_t st)
+{
+    if (T < 1 || I % 32) return 1;
+    const long long blocks = (long long)T * (I / 32);
+    swiglu_quant_kernel<<<(unsigned)((blocks + 7) / 8), 256, 0, st>>>(gu, (uint16_t*)out, T, I, lim);
+    return launch_status();
+}
+// reference qwen_moe.cu:101-111
+SPARK_API int qwen_moe_silu_mul(const void* g, const void* u, void* h, int n, hipStream_t st)
+{
+    if (n < 1) return 0;
+    silu_mul_kernel<<<(n + 255) / 256, 256, 0, st>>>((const float*)g, (const float*)u, (float*)h, n);
+    return launch_status();
+}
+SPARK_API int qwen_moe_gate_scale(const void* gl, int64_t ldg, int col, const void* d, void* out, int R, int N, hipStream_t st)
+{
+    if (R * N < 1) return 0;
+    gate_scale_kernel<<<(R * N + 255) / 256, 256, 0, st>>>((const float*)gl, ldg, col, (const float*)d, (float*)out, R, N);
+    return launch_status();
+}

@@ -1,0 +1,208 @@
+// Dense decode GEMVs on quantized weights, y[m, n] = x[m, :] . dequant(W)[n, :], m <= 8 rows, binary32 accumulation.
+//   MXFP4                     reference engine-rs/shim/ds41.cu:75-110,236
+//   FP8 E4M3, 32x32 E8M0      reference engine-rs/shim/ds41.cu:28-73,238-249
+//   FP8 E4M3, 128x128 fp32    reference reference/ds41/kernel.py:96-119 (the judged dense format)
+//   BF16 (router logits)      reference engine-rs/shim/ds41.cu:112-146,251-258
+// One wave64 per output row: every lane streams 16-byte pieces of the row (one piece never crosses a scale block),
+// converts them with the gfx950 packed converts to bf16 pairs (exact for E2M1 / E4M3) and accumulates bf16 x bf16
+// products in binary32 with v_dot2_f32_bf16; the block scale multiplies the piece's partial sum; lanes are summed with
+// a butterfly.  Activations are staged once per workgroup in LDS.
+#include "common.hpp"
+
+using namespace spk;
+
+typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr int GEMV_WAVES = 4, RPW = 4;
+
+__device__ __forceinline__ bf2 as_bf2(uint32_t v) { bf2 r; __builtin_memcpy(&r, &v, 4); return r; }
+
+// x [m, k] bf16 (row stride xs) -> LDS [m][k] (k elements per row, contiguous)
+__device__ __forceinline__ void stage_x(const uint16_t* __restrict__ x, int64_t xs, int64_t xoff, uint16_t* __restrict__ xl, int m, int k)
+{
+    const int n8 = k / 8;
+    for (int i = threadIdx.x; i < m * n8; i += blockDim.x) {
+        const int r = i / n8, c = (i % n8) * 8;
+        *(uint4*)(xl + r * k + c) = *(const uint4*)(x + r * xs + xoff + c);
+    }
+    __syncthreads();
+}
+
+// FMT 0: MXFP4 (16 bytes = 32 weights, E8M0 scale per row and 32), 1: FP8 + E8M0 per 32x32, 2: FP8 + fp32 per bs x bs.
+// A wave owns RPW consecutive rows and walks them together, so RPW 16-byte loads per lane are in flight at a time and
+// the activations staged in LDS serve GEMV_WAVES * RPW rows.
+template <int FMT, int M>
+__global__ __launch_bounds__(64 * GEMV_WAVES) void qgemv_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w, const void* __restrict__ sc,
+                                                                float* __restrict__ y, int m, int n, int k, int xs, int rpg, int bs)
+{
+    extern __shared__ uint16_t xl[];                      // [M][k] bf16
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wg_row0 = blockIdx.x * (GEMV_WAVES * RPW);
+    // grouped (block-diagonal) weights read input group row / rpg; a workgroup's rows share the group (rpg % 32 == 0)
+    const int64_t xoff = rpg ? (int64_t)(wg_row0 / rpg) * k : 0;
+    stage_x(x, xs, xoff, xl, m, k);
+    const int row0 = wg_row0 + wave * RPW;
+    if (row0 >= n) return;
+    constexpr int EPP = FMT == 0 ? 32 : 16;               // elements per 16-byte piece
+    const int64_t rb = FMT == 0 ? k / 2 : k;              // bytes per weight row
+    float acc[RPW][M];
+#pragma unroll
+    for (int i = 0; i < RPW; ++i)
+#pragma unroll
+        for (int r = 0; r < M; ++r) acc[i][r] = 0.f;
+    for (int c = lane * EPP; c < k; c += 64 * EPP) {
+        uint4 p[RPW];
+        float s[RPW];
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const int row = row0 + i < n ? row0 + i : n - 1;
+            p[i] = ld_stream16(w + (int64_t)row * rb + (FMT == 0 ? c / 2 : c));
+            if (FMT == 0) s[i] = e8m0_to_f32(((const uint8_t*)sc)[(int64_t)row * (k >> 5) + (c >> 5)]);
+            else if (FMT == 1) s[i] = e8m0_to_f32(((const uint8_t*)sc)[(int64_t)(row >> 5) * (k >> 5) + (c >> 5)]);
+            else s[i] = ((const float*)sc)[(int64_t)(row / bs) * ((k + bs - 1) / bs) + c / bs];
+        }
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const uint32_t pw[4] = {p[i].x, p[i].y, p[i].z, p[i].w};
+            bf2 wv[EPP / 2];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (FMT == 0) {
+                    wv[4 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 0);
+                    wv[4 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 1);
+                    wv[4 * j + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 2);
+                    wv[4 * j + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 3);
+                } else {
+                    wv[2 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, false);
+                    wv[2 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, true);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < M; ++r) {
+                if (r >= m) break;
+                const uint32_t* xp = (const uint32_t*)(xl + r * k + c);
+                float t = 0.f;
+#pragma unroll
+                for (int j = 0; j < EPP / 2; j += 4) {
+                    const uint4 xv = *(const uint4*)(xp + j);
+                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 0], as_bf2(xv.x), t, false);
+                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 1], as_bf2(xv.y), t, false);
+                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 2], as_bf2(xv.z), t, false);
+                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 3], as_bf2(xv.w), t, false);
+                }
+                acc[i][r] = __builtin_fmaf(t, s[i], acc[i][r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < RPW; ++i)
+#pragma unroll
+        for (int r = 0; r < M; ++r) {
+            if (r >= m) break;
+            const float v = wave_sum(acc[i][r]);
+            if (lane == 0 && row0 + i < n) y[(int64_t)r * n + row0 + i] = v;
+        }
+}
+
+template <int M>
+__global__ __launch_bounds__(64 * GEMV_WAVES) void bf16_gemv_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float* __restrict__ y,
+                                                                    int m, int n, int k)
+{
+    extern __shared__ uint16_t xl[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    stage_x(x, k, 0, xl, m, k);
+    const int row = blockIdx.x * GEMV_WAVES + wave;
+    if (row >= n) return;
+    const uint16_t* wr = w + (int64_t)row * k;
+    float acc[M];
+#pragma unroll
+    for (int r = 0; r < M; ++r) acc[r] = 0.f;
+    for (int c = lane * 8; c < k; c += 512) {
+        const uint4 p = ld_stream16(wr + c);
+#pragma unroll
+        for (int r = 0; r < M; ++r) {
+            if (r >= m) break;
+            const uint4 xv = *(const uint4*)(xl + r * k + c);
+            float t = acc[r];
+            t = __builtin_amdgcn_fdot2_f32_bf16(as_bf2(p.x), as_bf2(xv.x), t, false);
+            t = __builtin_amdgcn_fdot2_f32_bf16(as_bf2(p.y), as_bf2(xv.y), t, false);
+            t = __builtin_amdgcn_fdot2_f32_bf16(as_bf2(p.z), as_bf2(xv.z), t, false);
+            t = __builtin_amdgcn_fdot2_f32_bf16(as_bf2(p.w), as_bf2(xv.w), t, false);
+            acc[r] = t;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < M; ++r) {
+        if (r >= m) break;
+        const float v = wave_sum(acc[r]);
+        if (lane == 0) y[(int64_t)r * n + row] = v;
+    }
+}
+
+constexpr size_t LDS_MAX = 160 * 1024;
+
+template <int FMT>
+int launch_qgemv(const void* x, const void* w, const void* sc, float* y, int m, int n, int k, int xs, int rpg, int bs, hipStream_t st)
+{
+    const size_t sm = (size_t)m * k * 2;
+    if (sm > LDS_MAX) return 2;
+    const dim3 g((n + GEMV_WAVES * RPW - 1) / (GEMV_WAVES * RPW)), b(64 * GEMV_WAVES);
+#define QG(MM)                                                                                                                                   \
+    do {                                                                                                                                         \
+        static bool attr = hipFuncSetAttribute((const void*)qgemv_kernel<FMT, MM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX) == hipSuccess; \
+        if (!attr) return 3;                                                                                                                     \
+        qgemv_kernel<FMT, MM><<<g, b, sm, st>>>((const uint16_t*)x, (const uint8_t*)w, sc, y, m, n, k, xs, rpg, bs);                             \
+    } while (0)
+    switch (m) { case 1: QG(1); break; case 2: QG(2); break; case 3: case 4: QG(4); break; default: QG(8); }
+#undef QG
+    return launch_status();
+}
+
+}  // namespace
+
+// ================================================================ C ABI
+
+// reference ds41.cu:236: x bf16 [m, k], w E2M1 pairs [n, k/2], ws E8M0 [n, k/32], y f32 [m, n]; m <= 8, k % 32 == 0.
+// Here additionally k % 2048 == 0 or k <= 2048 is not required: any k % 32 == 0 works.
+SPARK_API int ds41_mxfp4_gemv(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, hipStream_t st)
+{
+    if (m < 1 || m > 8 || n < 1 || k < 32 || k % 32 != 0) return 1;
+    return launch_qgemv<0>(x, w, ws, y, m, n, k, k, 0, 0, st);
+}
+// reference ds41.cu:238-249: W E4M3 [n, k], scales E8M0 [ceil(n/32), k/32]; xs = input row stride, rpg = rows per group
+// of a block-diagonal weight (0: none)
+SPARK_API int ds41_fp8_gemv_ex(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, int xs, int rpg, hipStream_t st)
+{
+    if (m < 1 || m > 8 || n < 1 || k < 32 || k % 32 != 0 || (rpg && rpg % 32)) return 1;
+    return launch_qgemv<1>(x, w, ws, y, m, n, k, xs, rpg, 0, st);
+}
+SPARK_API int ds41_fp8_gemv(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, hipStream_t st)
+{
+    return ds41_fp8_gemv_ex(x, w, ws, y, m, n, k, k, 0, st);
+}
+// W E4M3 [n, k] with one binary32 scale per 128 x 128 block [ceil(n/128), ceil(k/128)], bf16 activations used as given.
+// No counterpart symbol in the reference shim: the format is that of reference/ds41/kernel.py:96-119 (fp8_gemm, block 128).
+SPARK_API int spark_fp8_block128_gemv(const void* x, const void* w, const float* scales, float* y, int m, int n, int k, hipStream_t st)
+{
+    if (m < 1 || m > 8 || n < 1 || k < 16 || k % 16 != 0) return 1;
+    return launch_qgemv<2>(x, w, scales, y, m, n, k, k, 0, 128, st);
+}
+// reference ds41.cu:251-258: W bf16 [n, k]
+SPARK_API int ds41_bf16_gemv(const void* x, const void* w, float* y, int m, int n, int k, hipStream_t st)
+{
+    if (m < 1 || m > 8 || n < 1 || k % 8 != 0) return 1;
+    const size_t sm = (size_t)m * k * 2;
+    if (sm > LDS_MAX) return 2;
+    const dim3 g((n + GEMV_WAVES - 1) / GEMV_WAVES), b(64 * GEMV_WAVES);
+#define BG(MM)                                                                                                                                   \
+    do {                                                                                                                                         \
+        static bool attr = hipFuncSetAttribute((const void*)bf16_gemv_kernel<MM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX) == hipSuccess; \
+        if (!attr) return 3;                                                                                                                     \
+        bf16_gemv_kernel<MM><<<g, b, sm, st>>>((const uint16_t*)x, (const uint16_t*)w, y, m, n, k);                                              \
+    } while (0)
+    switch (m) { case 1: BG(1); break; case 2: BG(2); break; case 3: case 4: BG(4); break; default: BG(8); }
+#undef BG
+    return launch_status();
+}

@@ -1,0 +1,360 @@
+// Routed EXL3 (4-bit trellis) experts for gfx950: Qwen-style (mul1 codebook) and GLM-style (mcg codebook, clamped SwiGLU).
+//
+//   out[r] = add[r] + sum_k (slot order) w[r][k] * ( act(x_r @ Wg_e, x_r @ Wu_e) @ Wd_e ),   e = idx[r][k]
+//   x @ W = had128( had128(x * suh) @ inner ) * svh                       (reference qwen_exl3.cuh:4-7)
+//
+// Semantics: reference engine-rs/shim/moe_exl3.cuh:1-13,204-228,272-285,935-1112,1512-1691 (moex::experts),
+// qwen_moe.cu:112-116, glm_moe.cu:10-14.  Expert table tab[9][E] of device pointers: gate_tr, up_tr, down_tr,
+// gate_suh, up_suh, down_suh, gate_svh, up_svh, down_svh (moe_exl3.cuh:8-9).
+//
+// MI355X design of the weight stream (the hot loop).  The reference decodes a tile into a 32-lane tensor-core fragment.
+// Here a wave64 takes eight adjacent 16x16 tiles (128 output columns of one k-tile, 1 KiB contiguous) per 128-bit load:
+// lane (j = lane / 8, m = lane % 8) holds words 4m..4m+3 of tile j = sequence positions 32m..32m+31 = all 16 k rows of
+// columns m and m + 8 of that tile.  So a lane owns two output columns outright: no cross-lane reduction over K, only
+// the three trailing nibbles of the previous word come from the neighbour lane.  States are cut out of the 64-bit
+// window with alignbit / bfe, decoded two at a time (packed fp16 codebook arithmetic) and accumulated with
+// v_dot2_f32_f16 against the Hadamard-transformed activations, which are wave-uniform and arrive as scalar loads.
+#include "common.hpp"
+#include "exl3_decode.hpp"
+
+using namespace spk;
+
+namespace {
+
+constexpr int EMAX = 1024;            // experts (one grouping thread each)
+constexpr int PMAX = 1024;            // routed pairs per call (decode / verify chains)
+constexpr int GV_WAVES = 4;
+
+enum XType { X_F32 = 0, X_F16 = 1, X_BF16 = 2 };
+
+struct Cfg {                          // runtime shape of one layer
+    int E, topk, H, I, cbk, act;      // act 0: silu(g) * u, 1: clamp (g <= 10, |u| <= 10) first
+    int xtype, wtype, itype;          // x: XType; route weights: 0 f32, 1 f16; indices: 0 int32, 1 int64
+};
+
+__device__ __forceinline__ float ld_x(const void* x, int xtype, int64_t i)
+{
+    if (xtype == X_F32) return ((const float*)x)[i];
+    if (xtype == X_F16) return f16_bits_to_f32(((const uint16_t*)x)[i]);
+    return bf16_to_f32(((const uint16_t*)x)[i]);
+}
+__device__ __forceinline__ int ld_idx(const void* idx, int itype, int i) { return itype ? (int)((const int64_t*)idx)[i] : ((const int*)idx)[i]; }
+__device__ __forceinline__ float ld_w(const void* w, int wtype, int i) { return wtype ? f16_bits_to_f32(((const uint16_t*)w)[i]) : ((const float*)w)[i]; }
+__device__ __forceinline__ float act_fn(int act, float a, float u)
+{
+    if (act == 1) { a = fminf(a, 10.0f); u = fminf(fmaxf(u, -10.0f), 10.0f); }
+    return a / (1.0f + __expf(-a)) * u;
+}
+
+// ---------------------------------------------------------------- grouping: stable counting sort of the pairs by expert
+// One workgroup, thread = expert.  Items of at most GR rows; rows ascending within an expert.
+// reference moe_exl3.cuh:961-1014 (prep_small_kernel).
+__global__ __launch_bounds__(EMAX) void prep_kernel(const void* __restrict__ idx, int itype, int R, int topk, int E, int GR, int* __restrict__ G,
+                                                   int* __restrict__ gexp, int* __restrict__ goff, int* __restrict__ gcnt, int* __restrict__ pairmap,
+                                                   int* __restrict__ prow, int* __restrict__ pexp)
+{
+    __shared__ int sidx[PMAX];
+    __shared__ int wr[16], wi[16];
+    const int e = threadIdx.x, n = R * topk;
+    for (int i = e; i < n; i += EMAX) sidx[i] = ld_idx(idx, itype, i);
+    __syncthreads();
+    int tot = 0;
+    if (e < E) for (int i = 0; i < n; ++i) tot += sidx[i] == e;
+    const int nit = (tot + GR - 1) / GR;
+    int ir = tot, ii = nit;
+    const int lane = e & 63, wv = e >> 6;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int a = __shfl_up(ir, o, 64), b = __shfl_up(ii, o, 64);
+        if (lane >= o) { ir += a; ii += b; }
+    }
+    if (lane == 63) { wr[wv] = ir; wi[wv] = ii; }
+    __syncthreads();
+    int rb = 0, ib = 0;
+    for (int w = 0; w < wv; ++w) { rb += wr[w]; ib += wi[w]; }
+    if (e == EMAX - 1) *G = ib + ii;
+    const int row0 = rb + ir - tot;
+    int it = ib + ii - nit;
+    for (int i = 0; i * GR < tot; ++i, ++it) { gexp[it] = e; goff[it] = row0 + i * GR; gcnt[it] = min(GR, tot - i * GR); }
+    int pos = row0;
+    if (tot)
+        for (int i = 0; i < n; ++i)
+            if (sidx[i] == e) { pairmap[i] = pos; prow[pos] = i / topk; pexp[pos] = e; ++pos; }
+}
+
+// ---------------------------------------------------------------- xh[t][row][K] = fp16(had128(x[src] * suh_t[e])); wave per (t, row, kb)
+// reference moe_exl3.cuh:204-228 (had_grouped_kernel), stage 1 (src = source row of the pair)
+__global__ __launch_bounds__(256) void had_kernel(const void* __restrict__ x, int xtype, int64_t ldx, const uint64_t* __restrict__ tab, int E, int suh_slot0,
+                                                  int T, int P, const int* __restrict__ prow, const int* __restrict__ pexp, int K, uint16_t* __restrict__ xh)
+{
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, lane = threadIdx.x & 63;
+    const int nb = K / 128;
+    const int kb = wave % nb, rest = wave / nb;
+    const int row = rest % P, t = rest / P;
+    if (t >= T) return;
+    const uint16_t* suh = (const uint16_t*)tab[(int64_t)(suh_slot0 + t) * E + pexp[row]];
+    const int64_t src = prow[row];
+    const int k = kb * 128 + lane * 2;
+    float v0 = ld_x(x, xtype, src * ldx + k) * f16_bits_to_f32(suh[k]);
+    float v1 = ld_x(x, xtype, src * ldx + k + 1) * f16_bits_to_f32(suh[k + 1]);
+    fwht128(v0, v1, lane);
+    uint16_t* d = xh + ((int64_t)t * P + row) * K + k;
+    d[0] = f32_to_f16_bits(v0);
+    d[1] = f32_to_f16_bits(v1);
+}
+
+// ---------------------------------------------------------------- the weight stream: partial GEMV of one item
+// grid (N / 128, S, T * Gmax), 4 waves.  Block (n-block nb, K slice s, matrix t, item g): rows goff[g] .. + gcnt[g] of
+// xh[t] times k-tiles [s kts, (s + 1) kts) of the expert's inner matrix, columns 128 nb .. + 127 -> part[s][t][row][N].
+// Waves interleave over the slice's k-tiles and are summed through LDS in wave order.
+__device__ __forceinline__ h2 as_h2(uint32_t v) { h2 r; __builtin_memcpy(&r, &v, 4); return r; }
+
+template <int CBK, int MR>
+__device__ __forceinline__ void tile_fma(const uint4 w, uint32_t prev, const uint32_t* __restrict__ xrow, int64_t ldx32, int rows, float (&acc)[MR][2])
+{
+    // decode this lane's 32 weights: word j holds k rows 2j, 2j+1, 2j+8, 2j+9 of column m (positions 0-3) and m+8 (4-7)
+    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+    h2 wd[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = ww[j], hi = j == 0 ? prev : ww[j - 1];
+        const uint32_t s0 = __builtin_amdgcn_alignbit(hi, lo, 28) & 0xffffu, s1 = __builtin_amdgcn_alignbit(hi, lo, 24) & 0xffffu;
+        const uint32_t s2 = __builtin_amdgcn_alignbit(hi, lo, 20) & 0xffffu, s3 = lo >> 16;
+        const uint32_t s4 = (lo >> 12) & 0xffffu, s5 = (lo >> 8) & 0xffffu, s6 = (lo >> 4) & 0xffffu, s7 = lo & 0xffffu;
+        wd[j][0] = cb_decode2<CBK>(s0, s1);
+        wd[j][1] = cb_decode2<CBK>(s2, s3);
+        wd[j][2] = cb_decode2<CBK>(s4, s5);
+        wd[j][3] = cb_decode2<CBK>(s6, s7);
+    }
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+        if (r >= rows) break;
+        const uint32_t* xp = xrow + r * ldx32;       // 8 packed fp16 pairs of this k-tile (wave-uniform address)
+        float a0 = acc[r][0], a1 = acc[r][1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const h2 xa = as_h2(xp[j]), xb = as_h2(xp[j + 4]);
+            a0 = __builtin_amdgcn_fdot2(wd[j][0], xa, a0, false);
+            a0 = __builtin_amdgcn_fdot2(wd[j][1], xb, a0, false);
+            a1 = __builtin_amdgcn_fdot2(wd[j][2], xa, a1, false);
+            a1 = __builtin_amdgcn_fdot2(wd[j][3], xb, a1, false);
+        }
+        acc[r][0] = a0; acc[r][1] = a1;
+    }
+}
+
+template <int CBK, int MR>
+__global__ __launch_bounds__(64 * GV_WAVES) void gemv_kernel(const uint16_t* __restrict__ xh, const uint64_t* __restrict__ tab, int E, int tr_slot0,
+                                                             const int* __restrict__ G, const int* __restrict__ gexp, const int* __restrict__ goff,
+                                                             const int* __restrict__ gcnt, int Gmax, int T, int P, int K, int N, int kts,
+                                                             float* __restrict__ part)
+{
+    __shared__ float red[GV_WAVES][MR][128];
+    const int tg = blockIdx.z, t = tg / Gmax, g = tg % Gmax;
+    if (g >= *G) return;
+    const int rows = gcnt[g];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int Nt = N / 16, nb = blockIdx.x, s = blockIdx.y;
+    const uint32_t* tr = (const uint32_t*)tab[(int64_t)(tr_slot0 + t) * E + gexp[g]];
+    const int64_t r0 = (int64_t)t * P + goff[g];
+    const uint32_t* xbase = (const uint32_t*)(xh + r0 * K);   // rows K fp16 = K/2 words apart
+    const int kt0 = s * kts, kt1 = min(K / 16, kt0 + kts);
+    float acc[MR][2];
+#pragma unroll
+    for (int r = 0; r < MR; ++r) { acc[r][0] = 0.f; acc[r][1] = 0.f; }
+    const int src = (lane & ~7) | ((lane + 7) & 7);           // lane holding the previous word of this lane's first word
+    // two k-tiles in flight per wave
+    for (int kt = kt0 + wave; kt < kt1; kt += 2 * GV_WAVES) {
+        const int ktb = kt + GV_WAVES;
+        const uint4 wa = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
+        uint4 wb = make_uint4(0u, 0u, 0u, 0u);
+        if (ktb < kt1) wb = ld_stream16(tr + ((int64_t)ktb * Nt + nb * 8) * 32 + lane * 4);
+        tile_fma<CBK, MR>(wa, __shfl(wa.w, src, 64), xbase + kt * 8, K / 2, rows, acc);
+        if (ktb < kt1) tile_fma<CBK, MR>(wb, __shfl(wb.w, src, 64), xbase + ktb * 8, K / 2, rows, acc);
+    }
+    const int j = lane >> 3, m = lane & 7;
+#pragma unroll
+    for (int r = 0; r < MR; ++r) { red[wave][r][16 * j + m] = acc[r][0]; red[wave][r][16 * j + m + 8] = acc[r][1]; }
+    __syncthreads();
+    float* out = part + (((int64_t)s * T * P) + r0) * N + nb * 128;
+    for (int i = threadIdx.x; i < rows * 128; i += 64 * GV_WAVES) {
+        const int r = i >> 7, c = i & 127;
+        float v = red[0][r][c];
+#pragma unroll
+        for (int w = 1; w < GV_WAVES; ++w) v += red[w][r][c];
+        out[(int64_t)r * N + c] = v;
+    }
+}
+
+// ---------------------------------------------------------------- mid: finish gate and up, act, down input transform
+// wave per (compact row, 128-block of I); reference moe_exl3.cuh:1019-1064
+__global__ __launch_bounds__(256) void mid_kernel(const float* __restrict__ part, int S, const uint64_t* __restrict__ tab, int E, int P, int I, int act,
+                                                  const int* __restrict__ pexp, uint16_t* __restrict__ xh2)
+{
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, lane = threadIdx.x & 63;
+    const int nb = I / 128, b = wave % nb, row = wave / nb;
+    if (row >= P) return;
+    const int e = pexp[row], n = b * 128 + 2 * lane;
+    float g[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const uint16_t* svh = (const uint16_t*)tab[(int64_t)(6 + t) * E + e];
+        float v0 = 0.f, v1 = 0.f;
+        for (int s = 0; s < S; ++s) {
+            const float* q = part + (((int64_t)s * 2 + t) * P + row) * I + n;
+            v0 += q[0]; v1 += q[1];
+        }
+        fwht128(v0, v1, lane);
+        g[t][0] = v0 * f16_bits_to_f32(svh[n]);
+        g[t][1] = v1 * f16_bits_to_f32(svh[n + 1]);
+    }
+    const uint16_t* suh = (const uint16_t*)tab[(int64_t)5 * E + e];
+    float v0 = act_fn(act, g[0][0], g[1][0]) * f16_bits_to_f32(suh[n]);
+    float v1 = act_fn(act, g[0][1], g[1][1]) * f16_bits_to_f32(suh[n + 1]);
+    fwht128(v0, v1, lane);
+    xh2[(int64_t)row * I + n] = f32_to_f16_bits(v0);
+    xh2[(int64_t)row * I + n + 1] = f32_to_f16_bits(v1);
+}
+
+// ---------------------------------------------------------------- finish of the down product + weighted slot-order sum
+// wave per (row r, 128-block of H): out[r] = add[r] + sum_k w[r][k] * (had128(sum_s part[s][pairmap[r][k]]) * svh_down[e_k])
+// reference moe_exl3.cuh:935-956,1084-1112,1380-1410
+__global__ __launch_bounds__(256) void finish_combine_kernel(const float* __restrict__ part, int S, const uint64_t* __restrict__ tab, int E, int P, int H,
+                                                             int topk, const int* __restrict__ pairmap, const int* __restrict__ pexp, const void* __restrict__ w,
+                                                             int wtype, const float* __restrict__ add, float* __restrict__ out, int R)
+{
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, lane = threadIdx.x & 63;
+    const int nb = H / 128, b = wave % nb, r = wave / nb;
+    if (r >= R) return;
+    const int n = b * 128 + 2 * lane;
+    float a0 = 0.f, a1 = 0.f;
+    for (int k = 0; k < topk; ++k) {
+        const int row = pairmap[r * topk + k];
+        const uint16_t* svh = (const uint16_t*)tab[(int64_t)8 * E + pexp[row]];
+        float v0 = 0.f, v1 = 0.f;
+        for (int s = 0; s < S; ++s) {
+            const float* q = part + ((int64_t)s * P + row) * H + n;
+            v0 += q[0]; v1 += q[1];
+        }
+        fwht128(v0, v1, lane);
+        const float wk = ld_w(w, wtype, r * topk + k);
+        a0 += wk * (v0 * f16_bits_to_f32(svh[n]));
+        a1 += wk * (v1 * f16_bits_to_f32(svh[n + 1]));
+    }
+    const float b0 = add ? add[(int64_t)r * H + n] : 0.f, b1 = add ? add[(int64_t)r * H + n + 1] : 0.f;
+    out[(int64_t)r * H + n] = b0 + a0;
+    out[(int64_t)r * H + n + 1] = b1 + a1;
+}
+
+// ---------------------------------------------------------------- host side
+inline int slices(int Kt, int nblocks) { int s = 1; while (s < 8 && nblocks * s < 768 && Kt / (s * 2) >= 8) s *= 2; return s; }
+
+struct Plan { int P, Gmax, S1, S2; size_t G, gexp, goff, gcnt, pairmap, prow, pexp, xh1, part, xh2, total; };
+inline Plan plan(const Cfg& c, int R)
+{
+    Plan p;
+    p.P = R * c.topk;
+    p.Gmax = p.P < c.E ? p.P : c.E;
+    p.S1 = slices(c.H / 16, (c.I / 128) * 2 * p.Gmax);
+    p.S2 = slices(c.I / 16, (c.H / 128) * p.Gmax);
+    size_t o = 0;
+    auto take = [&](size_t n) { const size_t q = o; o += align256(n); return q; };
+    p.G = take(16);
+    p.gexp = take(4 * (size_t)p.Gmax); p.goff = take(4 * (size_t)p.Gmax); p.gcnt = take(4 * (size_t)p.Gmax);
+    p.pairmap = take(4 * (size_t)p.P); p.prow = take(4 * (size_t)p.P); p.pexp = take(4 * (size_t)p.P);
+    p.xh1 = take(2 * (size_t)p.P * c.H * 2);
+    const size_t e1 = (size_t)p.S1 * 2 * p.P * c.I, e2 = (size_t)p.S2 * p.P * c.H;
+    p.part = take(4 * (e1 > e2 ? e1 : e2));
+    p.xh2 = take((size_t)p.P * c.I * 2);
+    p.total = o;
+    return p;
+}
+inline bool cfg_ok(const Cfg& c, int R)
+{
+    return R >= 1 && c.E >= 1 && c.E <= EMAX && c.topk >= 1 && c.topk <= 64 && (int64_t)R * c.topk <= PMAX && R <= 64 && c.H >= 128 && c.I >= 128 &&
+           c.H % 128 == 0 && c.I % 128 == 0 && (c.cbk == CB_MCG || c.cbk == CB_MUL1);
+}
+
+template <int CBK>
+void launch_gemv(const uint16_t* xh, const uint64_t* tab, int E, int slot0, const int* G, const int* gexp, const int* goff, const int* gcnt, int Gmax, int T,
+                 int P, int K, int N, int S, int maxrows, float* part, hipStream_t st)
+{
+    const dim3 grid(N / 128, S, T * Gmax), blk(64 * GV_WAVES);
+    const int kts = (K / 16 + S - 1) / S;
+    // one instantiation per row-count class of the call (items never hold more rows than the call has)
+    if (maxrows <= 1) gemv_kernel<CBK, 1><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
+    else if (maxrows <= 2) gemv_kernel<CBK, 2><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
+    else if (maxrows <= 4) gemv_kernel<CBK, 4><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
+    else if (maxrows <= 8) gemv_kernel<CBK, 8><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
+    else gemv_kernel<CBK, 16><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
+}
+
+int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
+            hipStream_t st)
+{
+    if (!cfg_ok(c, R)) return -1;
+    const Plan p = plan(c, R);
+    char* b = (char*)ws;
+    int* G = (int*)(b + p.G);
+    int *gexp = (int*)(b + p.gexp), *goff = (int*)(b + p.goff), *gcnt = (int*)(b + p.gcnt);
+    int *pairmap = (int*)(b + p.pairmap), *prow = (int*)(b + p.prow), *pexp = (int*)(b + p.pexp);
+    uint16_t* xh1 = (uint16_t*)(b + p.xh1);
+    float* part = (float*)(b + p.part);
+    uint16_t* xh2 = (uint16_t*)(b + p.xh2);
+    const uint64_t* tb = (const uint64_t*)tab;
+    const int GR = 16, maxrows = R < GR ? R : GR;
+    prep_kernel<<<1, EMAX, 0, st>>>(idx, c.itype, R, c.topk, c.E, GR, G, gexp, goff, gcnt, pairmap, prow, pexp);
+    int waves = 2 * p.P * (c.H / 128);
+    had_kernel<<<(waves + 3) / 4, 256, 0, st>>>(x, c.xtype, ldx, tb, c.E, 3, 2, p.P, prow, pexp, c.H, xh1);
+    if (c.cbk == CB_MCG) launch_gemv<CB_MCG>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, p.S1, maxrows, part, st);
+    else launch_gemv<CB_MUL1>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, p.S1, maxrows, part, st);
+    waves = p.P * (c.I / 128);
+    mid_kernel<<<(waves + 3) / 4, 256, 0, st>>>(part, p.S1, tb, c.E, p.P, c.I, c.act, pexp, xh2);
+    if (c.cbk == CB_MCG) launch_gemv<CB_MCG>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, p.S2, maxrows, part, st);
+    else launch_gemv<CB_MUL1>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, p.S2, maxrows, part, st);
+    waves = R * (c.H / 128);
+    finish_combine_kernel<<<(waves + 3) / 4, 256, 0, st>>>(part, p.S2, tb, c.E, p.P, c.H, c.topk, pairmap, pexp, w, c.wtype, (const float*)add, (float*)out, R);
+    return launch_status();
+}
+
+const Cfg QWEN{512, 10, 2560, 640, CB_MUL1, 0, X_F32, 0, 0};
+const Cfg GLM{288, 8, 4096, 1024, CB_MCG, 1, X_F16, 1, 1};
+
+}  // namespace
+
+// ================================================================ C ABI
+
+// Runtime-sized entry (no reference counterpart symbol): x [R, H] of xtype (0 f32, 1 f16, 2 bf16), row stride ldx;
+// idx [R, topk] int32 (itype 0) or int64 (1); w [R, topk] f32 (wtype 0) or f16 (1); tab u64 [9][E]; codebook 2 = mul1,
+// 1 = mcg; act 0 = silu(g) u, 1 = clamped; add / out f32 [R, H].  4-bit trellis, R <= 64 rows.
+SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk)
+{
+    const Cfg c{E, topk, H, I, CB_MUL1, 0, 0, 0, 0};
+    if (!cfg_ok(c, R)) return 0;
+    return plan(c, R).total;
+}
+SPARK_API int spark_exl3_moe(const void* x, int xtype, int64_t ldx, int R, const void* idx, int itype, const void* w, int wtype, const void* tab,
+                             const void* add, void* out, void* ws, int H, int I, int E, int topk, int codebook, int act, hipStream_t st)
+{
+    const Cfg c{E, topk, H, I, codebook, act, xtype, wtype, itype};
+    return experts(c, x, ldx, R, idx, w, tab, add, out, ws, st);
+}
+// reference qwen_moe.cu:112-116: x f32 [R, 2560], idx i32 / w f32 [R, 10], tab u64 [9][512], out f32 [R, 2560]; S is the
+// reference's K-slice hint (the slice count is chosen from the shape here)
+SPARK_API size_t qwen_moe_ws_bytes(int R, int S) { (void)S; return spark_exl3_moe_ws_bytes(R, QWEN.H, QWEN.I, QWEN.E, QWEN.topk); }
+SPARK_API int qwen_moe_experts(const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws, int S,
+                               hipStream_t st)
+{
+    (void)S;
+    return experts(QWEN, x, ldx, R, idx, w, tab, add, out, ws, st);
+}
+// reference glm_moe.cu:6-24: x f16 [R, 4096], idx i64 / w f16 [R, 8], tab u64 [10|11][288] (rows 0-8 as above), mcg codebook,
+// clamped SwiGLU.  suh0 (shared gate/up input scales) is a prefill shortcut and is not needed; kmask must be 1 << 4.
+SPARK_API size_t glm_moe_ws_bytes(int R, int S) { (void)S; return spark_exl3_moe_ws_bytes(R, GLM.H, GLM.I, GLM.E, GLM.topk); }
+SPARK_API int glm_moe_experts(const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws, int S,
+                              const void* suh0, int kmask, hipStream_t st)
+{
+    (void)S; (void)suh0;
+    if (kmask != (1 << 4)) return -4;                          // mixed trellis widths: not built
+    return experts(GLM, x, ldx, R, idx, w, tab, add, out, ws, st);
+}

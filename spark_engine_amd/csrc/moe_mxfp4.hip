@@ -1,0 +1,514 @@
+// Routed MXFP4 experts (DeepSeek-style MoE layer) for gfx950.
+//
+//   y[r] = add[r] + sum_shared expert_s(x[r]) + sum_k (slot order) w2_e . q(bf16(silu(min(bf16(w1_e . xq_r), 10)) *
+//          clamp(bf16(w3_e . xq_r), +-10) * rw[r][k]))          e = idx[r][k], q = act_quant (E4M3 + UE8M0 per 32)
+//
+// Semantics: reference engine-rs/shim/ds41_moe.cu:1-24 and ds41_mx.cu:1-16,95-317,1436-1523 (ds41_moe_mx_ex),
+// reference engine-rs/src/ds41/kern.rs:1116-1133 (moe_ref).
+//
+// MI355X design.  The products run on the block-scaled matrix unit, v_mfma_scale_f32_16x16x128_f8f6f4 with A = 16 weight
+// rows in E2M1 (one E8M0 scale per lane = per row and 32-block, exactly the stored format) and B = up to 16 token rows in
+// E4M3 with their UE8M0 scales.  A lane's A operand is 16 contiguous bytes of the weight stream, so the packed weights go
+// from the 128-bit load straight into the instruction with no unpacking; products and scales are exact, only the
+// summation order differs from a dequantize + FP32 matmul.
+// Operand layout measured on gfx950: A/B lane l = row/column l % 16, K group g = l / 16.  An E2M1 operand holds
+// k = 32 g + e (nibble e of its 16 bytes); an E4M3 operand holds k = 16 g + e in registers 0-3 and k = 64 + 16 g + e in
+// registers 4-7; the scale byte of lane l applies to logical block g (k in [32 g, 32 g + 32)); D lane l = column l % 16,
+// rows 4 (l / 16) + {0..3}.
+//
+// Weight storage ("T16" records, written once by spark_mxfp4_prepack): per 16 rows and 512-wide K group one record of
+// 4352 bytes = 4 steps x (64 lanes x 16 bytes of codes) + 64 lanes x 4 scale bytes (byte s = step s).  A wave streams a
+// record with four 16-byte loads and one 4-byte load per lane, all contiguous.
+#include "common.hpp"
+
+using namespace spk;
+
+namespace {
+
+struct Item { int e, off, n, pad; };
+
+constexpr int REC = 4352;              // bytes per T16 record
+constexpr int EMAXG = 2048;            // experts the grouping kernel can hold
+constexpr int UP_WAVES = 8, DN_WAVES = 4;
+
+enum Layout { L_T16 = 0, L_NATURAL = 1, L_PACK8 = 2, L_MX8 = 3 };
+
+struct WMat {                          // one stacked weight matrix [E, rows, K]
+    const uint8_t* w;
+    const uint8_t* s;
+    int rows, K;                       // per expert
+};
+
+// ---- A operand: the 4 steps of K group kg of the 16 rows starting at row0 (row0 % 16 == 0) of expert e
+template <int LAYOUT>
+__device__ __forceinline__ void load_group(const WMat& m, int e, int row0, int kg, int lane, v4i (&c)[4], uint32_t& sc4)
+{
+    const int r = lane & 15, g = lane >> 4, steps = m.K >> 7, nkg = (steps + 3) >> 2;
+    if constexpr (LAYOUT == L_T16) {
+        const int64_t tile = ((int64_t)e * m.rows + row0) >> 4;
+        const uint8_t* rec = m.w + (tile * nkg + kg) * REC;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { const uint4 v = ld_stream16(rec + s * 1024 + lane * 16); c[s] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}; }
+        sc4 = __builtin_nontemporal_load((const uint32_t*)(rec + 4096 + lane * 4));
+    } else {
+        sc4 = 0x7f7f7f7fu;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int step = kg * 4 + s;
+            c[s] = v4i{0, 0, 0, 0};
+            if (step >= steps) continue;
+            const int64_t row = (int64_t)e * m.rows + row0 + r;
+            uint32_t sb;
+            if constexpr (LAYOUT == L_NATURAL) {
+                const uint4 v = ld_stream16(m.w + row * (m.K >> 1) + step * 64 + g * 16);
+                c[s] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                sb = m.s[row * (m.K >> 5) + step * 4 + g];
+            } else if constexpr (LAYOUT == L_PACK8) {      // [rows/8][K/128][8][4][16], scales [rows/8][K/128][8][4]
+                const int64_t t8 = row >> 3;
+                const uint4 v = ld_stream16(m.w + (t8 * steps + step) * 512 + (row & 7) * 64 + g * 16);
+                c[s] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                sb = m.s[(t8 * steps + step) * 32 + (row & 7) * 4 + g];
+            } else {                                        // L_MX8: [rows/8][K/128][8][4 q][4 b][4]
+                const int64_t t8 = row >> 3;
+                const uint32_t* p = (const uint32_t*)(m.w + (t8 * steps + step) * 512 + (row & 7) * 64 + g * 4);
+                c[s] = v4i{(int)p[0], (int)p[4], (int)p[8], (int)p[12]};
+                sb = m.s[(t8 * steps + step) * 32 + (row & 7) * 4 + g];
+            }
+            sc4 = (sc4 & ~(0xffu << (8 * s))) | (sb << (8 * s));
+        }
+    }
+}
+
+// ---- B operand of one step: E4M3 bytes of row `q` (row stride K) + its UE8M0 scales (row stride K/32)
+__device__ __forceinline__ void load_b(const uint8_t* __restrict__ q, const uint8_t* __restrict__ qs, int step, int lane, v8i& b, uint32_t& sb)
+{
+    const int g = lane >> 4;
+    const uint4 lo = *(const uint4*)(q + step * 128 + 16 * g);
+    const uint4 hi = *(const uint4*)(q + step * 128 + 64 + 16 * g);
+    b = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    sb = qs[step * 4 + g];
+}
+
+template <int OPSEL>
+__device__ __forceinline__ v4f mfma_step(const v4i& a, const v8i& b, v4f acc, uint32_t sa, uint32_t sb)
+{
+    const v8i a8 = v8i{a.x, a.y, a.z, a.w, 0, 0, 0, 0};
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b, acc, 4 /*A: E2M1*/, 0 /*B: E4M3*/, OPSEL, (int)sa, 0, (int)sb);
+}
+__device__ __forceinline__ v4f mfma_group_step(int s, const v4i& a, const v8i& b, v4f acc, uint32_t sa4, uint32_t sb)
+{
+    switch (s) {
+        case 0: return mfma_step<0>(a, b, acc, sa4, sb);
+        case 1: return mfma_step<1>(a, b, acc, sa4, sb);
+        case 2: return mfma_step<2>(a, b, acc, sa4, sb);
+        default: return mfma_step<3>(a, b, acc, sa4, sb);
+    }
+}
+
+// ---------------------------------------------------------------- grouping of the (row, expert) pairs by expert
+// Pairs per row: topk routed (idx, rw) followed by n_shared shared experts (ids E .. E + n_shared - 1, weight 1).
+// Items = at most GR compact rows of one expert.  One workgroup.  reference ds41_mx.cu:95-125.
+__global__ __launch_bounds__(1024) void group_kernel(const int64_t* __restrict__ idx, const float* __restrict__ rw, int R, int topk, int n_shared, int E,
+                                                    int GR, int* __restrict__ G, Item* __restrict__ items, int* __restrict__ pairmap, int* __restrict__ prow,
+                                                    float* __restrict__ pw, int* __restrict__ counters, int ncounters)
+{
+    __shared__ int cnt[EMAXG], fill[EMAXG], eoff[EMAXG], ioff[EMAXG];
+    __shared__ int wsum[2][16];
+    const int ET = E + n_shared, TT = topk + n_shared, P = R * TT, tid = threadIdx.x;
+    for (int i = tid; i < ncounters; i += 1024) counters[i] = 0;
+    for (int e = tid; e < ET; e += 1024) { cnt[e] = 0; fill[e] = 0; }
+    __syncthreads();
+    for (int p = tid; p < P; p += 1024) {
+        const int r = p / TT, k = p % TT;
+        const int e = k < topk ? (int)idx[(int64_t)r * topk + k] : E + (k - topk);
+        atomicAdd(&cnt[e], 1);
+    }
+    __syncthreads();
+    // exclusive scans of rows and items over the experts (two experts per thread)
+    int c0 = 0, c1 = 0;
+    if (2 * tid < ET) c0 = cnt[2 * tid];
+    if (2 * tid + 1 < ET) c1 = cnt[2 * tid + 1];
+    const int n0 = (c0 + GR - 1) / GR, n1 = (c1 + GR - 1) / GR;
+    int rs = c0 + c1, is = n0 + n1;
+    const int lane = tid & 63, wv = tid >> 6;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int a = __shfl_up(rs, o, 64), b = __shfl_up(is, o, 64);
+        if (lane >= o) { rs += a; is += b; }
+    }
+    if (lane == 63) { wsum[0][wv] = rs; wsum[1][wv] = is; }
+    __syncthreads();
+    int rbase = 0, ibase = 0;
+    for (int w = 0; w < wv; ++w) { rbase += wsum[0][w]; ibase += wsum[1][w]; }
+    const int rex = rbase + rs - (c0 + c1), iex = ibase + is - (n0 + n1);
+    if (2 * tid < ET) { eoff[2 * tid] = rex; ioff[2 * tid] = iex; }
+    if (2 * tid + 1 < ET) { eoff[2 * tid + 1] = rex + c0; ioff[2 * tid + 1] = iex + n0; }
+    if (tid == 1023) *G = ibase + is;
+    __syncthreads();
+    for (int e = tid; e < ET; e += 1024) {
+        const int c = cnt[e];
+        for (int j = 0; j * GR < c; ++j) items[ioff[e] + j] = Item{e, eoff[e] + j * GR, min(GR, c - j * GR), 0};
+    }
+    for (int p = tid; p < P; p += 1024) {
+        const int r = p / TT, k = p % TT;
+        const int e = k < topk ? (int)idx[(int64_t)r * topk + k] : E + (k - topk);
+        const int pos = eoff[e] + atomicAdd(&fill[e], 1);
+        pairmap[p] = pos;
+        prow[pos] = p;
+        pw[pos] = k < topk ? rw[(int64_t)r * topk + k] : 1.0f;
+    }
+}
+
+// ---------------------------------------------------------------- gate / up + SwiGLU + act_quant -> hq [P, I], hs [P, I/32]
+// grid (I / 32, Gmax), 8 waves: wave w takes K groups w, w + 8, ... of the 32 gate and 32 up rows j0 .. j0 + 31 for the
+// item's rows (16 per MFMA column group); the partial tiles are summed through LDS in wave order.
+template <int LAYOUT>
+__global__ __launch_bounds__(64 * UP_WAVES) void up_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, WMat w1, WMat w3, int H, int I, int TT,
+                                                           const int* __restrict__ G, const Item* __restrict__ items, const int* __restrict__ prow,
+                                                           const float* __restrict__ pw, uint8_t* __restrict__ hq, uint8_t* __restrict__ hs)
+{
+    __shared__ float red[UP_WAVES][4][4][64];      // [wave][tile: g0 g1 u0 u1][v][lane]
+    __shared__ float amx[UP_WAVES][16];
+    if ((int)blockIdx.y >= *G) return;
+    const Item it = items[blockIdx.y];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, rg = lane >> 4;
+    const int j0 = blockIdx.x * 32;
+    const int steps = H >> 7, nkg = (steps + 3) >> 2;
+    for (int cg = 0; cg * 16 < it.n; ++cg) {
+        const int rr = cg * 16 + c;                // compact row of this lane's column within the item
+        const bool valid = rr < it.n;
+        const int pos = it.off + (valid ? rr : 0);
+        const int tok = prow[pos] / TT;
+        const uint8_t* xr = xq + (int64_t)tok * H;
+        const uint8_t* xsr = xs + (int64_t)tok * (H >> 5);
+        v4f acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) { acc[t] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(acc[t])); }
+        for (int kg = wave; kg < nkg; kg += UP_WAVES) {
+            v4i a[4][4];
+            uint32_t sa[4];
+            load_group<LAYOUT>(w1, it.e, j0, kg, lane, a[0], sa[0]);
+            load_group<LAYOUT>(w1, it.e, j0 + 16, kg, lane, a[1], sa[1]);
+            load_group<LAYOUT>(w3, it.e, j0, kg, lane, a[2], sa[2]);
+            load_group<LAYOUT>(w3, it.e, j0 + 16, kg, lane, a[3], sa[3]);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int step = kg * 4 + s;
+                if (step >= steps) break;
+                v8i b; uint32_t sb;
+                load_b(xr, xsr, step, lane, b, sb);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[t] = mfma_group_step(s, a[t][s], b, acc[t], sa[t], sb);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][t][v][lane] = acc[t][v];
+        __syncthreads();
+        // epilogue: thread (wave = (tp, v), lane = (c, rg)) owns feature j0 + 16 tp + 4 rg + v of column c
+        const int tp = wave >> 2, v = wave & 3;
+        float gsum = 0.f, usum = 0.f;
+#pragma unroll
+        for (int w = 0; w < UP_WAVES; ++w) { gsum += red[w][tp][v][lane]; usum += red[w][2 + tp][v][lane]; }
+        const float wgt = valid ? pw[pos] : 0.f;
+        const float gt = fminf(bf16_round(gsum), 10.f);
+        const float up = fminf(fmaxf(bf16_round(usum), -10.f), 10.f);
+        const float yv = bf16_round(silu(gt) * up * wgt);
+        float am = fabsf(yv);
+        am = fmaxf(am, __shfl_xor(am, 16, 64));
+        am = fmaxf(am, __shfl_xor(am, 32, 64));
+        if (rg == 0) amx[wave][c] = am;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < UP_WAVES; ++w) am = fmaxf(am, amx[w][c]);
+        const uint32_t e = aq_scale(am);
+        if (valid) {
+            hq[(int64_t)pos * I + j0 + 16 * tp + 4 * rg + v] = (uint8_t)aq_byte(yv, e);
+            if (wave == 0 && rg == 0) hs[(int64_t)pos * (I >> 5) + (j0 >> 5)] = (uint8_t)e;
+        }
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------- down: out [P, H] = h . w2_e^T
+// grid (H / 32, Gmax), 4 waves: wave w takes K groups w, w + 4, ... of output rows n0 .. n0 + 31.
+template <int LAYOUT>
+__global__ __launch_bounds__(64 * DN_WAVES) void down_kernel(const uint8_t* __restrict__ hq, const uint8_t* __restrict__ hs, WMat w2, int H, int I,
+                                                             const int* __restrict__ G, const Item* __restrict__ items, float* __restrict__ out)
+{
+    __shared__ float red[DN_WAVES][2][4][64];
+    if ((int)blockIdx.y >= *G) return;
+    const Item it = items[blockIdx.y];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15;
+    const int n0 = blockIdx.x * 32;
+    const int steps = I >> 7, nkg = (steps + 3) >> 2;
+    for (int cg = 0; cg * 16 < it.n; ++cg) {
+        const int rr = cg * 16 + c;
+        const int pos = it.off + (rr < it.n ? rr : 0);
+        const uint8_t* hr = hq + (int64_t)pos * I;
+        const uint8_t* hsr = hs + (int64_t)pos * (I >> 5);
+        v4f acc[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) { acc[t] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(acc[t])); }
+        for (int kg = wave; kg < nkg; kg += DN_WAVES) {
+            v4i a[2][4];
+            uint32_t sa[2];
+            load_group<LAYOUT>(w2, it.e, n0, kg, lane, a[0], sa[0]);
+            load_group<LAYOUT>(w2, it.e, n0 + 16, kg, lane, a[1], sa[1]);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int step = kg * 4 + s;
+                if (step >= steps) break;
+                v8i b; uint32_t sb;
+                load_b(hr, hsr, step, lane, b, sb);
+#pragma unroll
+                for (int t = 0; t < 2; ++t) acc[t] = mfma_group_step(s, a[t][s], b, acc[t], sa[t], sb);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][t][v][lane] = acc[t][v];
+        __syncthreads();
+        // thread (wave = v, lane) sums both tiles' element v
+        const int v = wave, rg = lane >> 4;
+        if (rr < it.n) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < DN_WAVES; ++w) s += red[w][t][v][lane];
+                out[(int64_t)pos * H + n0 + 16 * t + 4 * rg + v] = s;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// y[r] = (add[r] + sum of the shared experts' outputs) + (sum_k routed out[pairmap[r, k]], k ascending)
+// reference ds41_mx.cu:302-317
+__global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ out, const int* __restrict__ pairmap, const float* __restrict__ add,
+                                                      float* __restrict__ y, int nr, int H, int topk, int n_shared)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int h4 = H >> 2;
+    if (i >= (int64_t)nr * h4) return;
+    const int r = (int)(i / h4), col = (int)(i % h4) * 4, TT = topk + n_shared;
+    float4 acc = add ? *(const float4*)(add + (int64_t)r * H + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k = topk; k < TT; ++k) {
+        const float4 v = *(const float4*)(out + (int64_t)pairmap[r * TT + k] * H + col);
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    }
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k = 0; k < topk; ++k) {
+        const float4 v = *(const float4*)(out + (int64_t)pairmap[r * TT + k] * H + col);
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    acc.x += s.x; acc.y += s.y; acc.z += s.z; acc.w += s.w;
+    *(float4*)(y + (int64_t)r * H + col) = acc;
+}
+
+// ---------------------------------------------------------------- natural layout -> T16 records
+// w [rows_total, K/2], s [rows_total, K/32] (rows_total % 16 == 0, K % 128 == 0); one thread per (tile, K group, lane).
+__global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ s, uint8_t* __restrict__ out, int64_t tiles, int K)
+{
+    const int steps = K >> 7, nkg = (steps + 3) >> 2;
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= tiles * nkg * 64) return;
+    const int lane = (int)(gid & 63);
+    const int64_t rec = gid >> 6;
+    const int kg = (int)(rec % nkg);
+    const int64_t tile = rec / nkg, row = tile * 16 + (lane & 15);
+    const int g = lane >> 4;
+    uint8_t* o = out + rec * REC;
+    uint32_t sc4 = 0x7f7f7f7fu;
+    for (int st = 0; st < 4; ++st) {
+        const int step = kg * 4 + st;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (step < steps) {
+            v = *(const uint4*)(w + row * (K >> 1) + step * 64 + g * 16);
+            sc4 = (sc4 & ~(0xffu << (8 * st))) | ((uint32_t)s[row * (K >> 5) + step * 4 + g] << (8 * st));
+        }
+        *(uint4*)(o + st * 1024 + lane * 16) = v;
+    }
+    *(uint32_t*)(o + 4096 + lane * 4) = sc4;
+}
+
+// ---------------------------------------------------------------- host side
+inline int gr_of(int R) { return R <= 16 ? 16 : 64; }
+inline int gmax_of(int R, int TT, int ET)
+{
+    const int64_t P = (int64_t)R * TT;
+    return (int)((P < ET ? P : ET) + P / gr_of(R) + 1);
+}
+struct WsLayout {
+    size_t G, items, pairmap, prow, pw, hq, hs, out, total;
+};
+inline WsLayout ws_layout(int R, int H, int I, int TT, int ET)
+{
+    const size_t P = (size_t)R * TT;
+    WsLayout l;
+    size_t o = 0;
+    l.G = o; o += align256(16 + 64 * 4);                       // G + a few counters
+    l.items = o; o += align256(sizeof(Item) * (size_t)gmax_of(R, TT, ET));
+    l.pairmap = o; o += align256(4 * P);
+    l.prow = o; o += align256(4 * P);
+    l.pw = o; o += align256(4 * P);
+    l.hq = o; o += align256(P * I);
+    l.hs = o; o += align256(P * I / 32);
+    l.out = o; o += align256(4 * P * H);
+    l.total = o;
+    return l;
+}
+
+template <int LAYOUT>
+int moe_launch(const uint8_t* xq, const uint8_t* xs, int R, const int64_t* idx, const float* rw, const uint8_t* w1, const uint8_t* s1, const uint8_t* w3,
+               const uint8_t* s3, const uint8_t* w2, const uint8_t* s2, int H, int I, int topk, int E, int n_shared, const float* add, float* y, void* ws,
+               int skip_combine, hipStream_t st)
+{
+    const int TT = topk + n_shared, ET = E + n_shared, GR = gr_of(R), Gm = gmax_of(R, TT, ET);
+    const WsLayout l = ws_layout(R, H, I, TT, ET);
+    char* base = (char*)ws;
+    int* G = (int*)(base + l.G);
+    Item* items = (Item*)(base + l.items);
+    int* pairmap = (int*)(base + l.pairmap);
+    int* prow = (int*)(base + l.prow);
+    float* pw = (float*)(base + l.pw);
+    uint8_t* hq = (uint8_t*)(base + l.hq);
+    uint8_t* hs = (uint8_t*)(base + l.hs);
+    float* out = (float*)(base + l.out);
+    group_kernel<<<1, 1024, 0, st>>>(idx, rw, R, topk, n_shared, E, GR, G, items, pairmap, prow, pw, G + 4, 64);
+    const WMat m1{w1, s1, I, H}, m3{w3, s3, I, H}, m2{w2, s2, H, I};
+    up_kernel<LAYOUT><<<dim3(I / 32, Gm), 64 * UP_WAVES, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
+    down_kernel<LAYOUT><<<dim3(H / 32, Gm), 64 * DN_WAVES, 0, st>>>(hq, hs, m2, H, I, G, items, out);
+    if (!skip_combine) {
+        const int64_t n4 = (int64_t)R * (H / 4);
+        combine_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(out, pairmap, add, y, R, H, topk, n_shared);
+    }
+    return launch_status();
+}
+
+inline bool shapes_ok(int R, int H, int I, int topk, int E, int n_shared)
+{
+    return R >= 1 && H >= 128 && I >= 128 && H % 128 == 0 && I % 128 == 0 && topk >= 1 && n_shared >= 0 && E >= 1 && E + n_shared <= EMAXG;
+}
+
+int g_s2 = 0;          // scale blobs handed to the ds41_moe_mx* symbols are 2-bit coded (reference ds41_mx.cu:1304)
+
+}  // namespace
+
+// ================================================================ C ABI: runtime-sized entry points (no reference counterpart symbol)
+
+// bytes of one stacked matrix [rows_total, K] in T16 records
+SPARK_API size_t spark_mxfp4_packed_bytes(long long rows_total, int K)
+{
+    if (rows_total < 16 || rows_total % 16 || K < 128 || K % 128) return 0;
+    return (size_t)(rows_total / 16) * ((K / 128 + 3) / 4) * REC;
+}
+// natural layout (w [rows_total, K/2], s [rows_total, K/32], device) -> T16 records (device)
+SPARK_API int spark_mxfp4_prepack(const void* w, const void* s, void* packed, long long rows_total, int K, hipStream_t st)
+{
+    if (rows_total < 16 || rows_total % 16 || K < 128 || K % 128) return 1;
+    const int64_t tiles = rows_total / 16, n = tiles * ((K / 128 + 3) / 4) * 64;
+    prepack_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((const uint8_t*)w, (const uint8_t*)s, (uint8_t*)packed, tiles, K);
+    return launch_status();
+}
+SPARK_API size_t spark_mxfp4_moe_ws_bytes(int R, int H, int I, int topk, int E, int n_shared)
+{
+    if (!shapes_ok(R, H, I, topk, E, n_shared)) return 0;
+    return ws_layout(R, H, I, topk + n_shared, E + n_shared).total;
+}
+// xq [R, H] E4M3 + xs [R, H/32] UE8M0 (act_quant of x); idx int64 / rw f32 [R, topk]; stacked weights of E + n_shared
+// experts: layout 0 = T16 records (s* unused), 1 = natural [E, rows, K/2] + [E, rows, K/32]; the n_shared experts after
+// the E routed ones run on every row with weight 1; add [R, H] f32 or null; y [R, H] f32.
+SPARK_API int spark_mxfp4_moe_q(const void* xq, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3,
+                                const void* s3, const void* w2, const void* s2, int layout, int H, int I, int topk, int E, int n_shared, const float* add,
+                                float* y, void* ws, hipStream_t st)
+{
+    if (!shapes_ok(R, H, I, topk, E, n_shared)) return 1;
+    if (layout == L_T16)
+        return moe_launch<L_T16>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, nullptr, (const uint8_t*)w3, nullptr, (const uint8_t*)w2,
+                                 nullptr, H, I, topk, E, n_shared, add, y, ws, 0, st);
+    if (layout == L_NATURAL)
+        return moe_launch<L_NATURAL>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3,
+                                     (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, H, I, topk, E, n_shared, add, y, ws, 0, st);
+    return 1;
+}
+extern "C" int ds41_act_quant_fp8(const void* x, void* q, void* s, long long numel, hipStream_t st);
+// x bf16 [R, H]: act_quant per 32 first (scratch xq, xs from the caller: R*H and R*H/32 bytes), then spark_mxfp4_moe_q
+SPARK_API int spark_mxfp4_moe(const void* x, void* xq, void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3,
+                              const void* s3, const void* w2, const void* s2, int layout, int H, int I, int topk, int E, int n_shared, const float* add, float* y,
+                              void* ws, hipStream_t st)
+{
+    if (!shapes_ok(R, H, I, topk, E, n_shared)) return 1;
+    const int rc = ds41_act_quant_fp8(x, xq, xs, (long long)R * H, st);
+    if (rc) return rc;
+    return spark_mxfp4_moe_q(xq, xs, R, idx, rw, w1, s1, w3, s3, w2, s2, layout, H, I, topk, E, n_shared, add, y, ws, st);
+}
+
+// ================================================================ C ABI: the reference's symbols (hidden size 5120)
+// reference ds41_mx.cu:1303-1523, ds41_moe.cu:257-292; Rust declarations engine-rs/src/ds41/kern.rs:5-80.
+namespace { constexpr int DS41_H = 5120; }
+
+SPARK_API void ds41_moe_mx_set_s2(int on) { g_s2 = on; }
+SPARK_API int ds41_moe_mx_get_s2() { return g_s2; }
+SPARK_API void ds41_moe_gr16_max(int) {}                       // row-count switch of the reference's item size: one kernel family here
+SPARK_API int ds41_moe_mx_col_passes(int, int, int) { return 1; }
+SPARK_API int ds41_moe_mx_pair_b16(int, int, int) { return 0; }
+SPARK_API size_t ds41_moe_mx_ws_bytes(int R, int I, int topk, int E) { return spark_mxfp4_moe_ws_bytes(R, DS41_H, I, topk, E, 0); }
+SPARK_API size_t ds41_moe_ws_bytes(int R, int I, int topk, int E)
+{
+    return spark_mxfp4_moe_ws_bytes(R, DS41_H, I, topk, E, 0) + align256((size_t)R * DS41_H) + align256((size_t)R * DS41_H / 32);
+}
+// weights in the reference's "mx" tile layout (kern.rs:728-734 moe_pack_mx), raw scales [tiles][K/128][8][4]
+SPARK_API int ds41_moe_mx_ex(const void* xq, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3,
+                             const void* s3, const void* w2, const void* s2, int I, const float* add, float* y, void* ws, int topk, int E, int skip_combine,
+                             hipStream_t st)
+{
+    if (R < 1 || I % 128 != 0 || E > 384 || topk < 1) return 1;
+    if (g_s2) return 5;                                        // 2-bit coded scale blobs are not decoded here
+    return moe_launch<L_MX8>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3, (const uint8_t*)s3,
+                             (const uint8_t*)w2, (const uint8_t*)s2, DS41_H, I, topk, E, 0, add, y, ws, skip_combine, st);
+}
+SPARK_API int ds41_moe_mx(const void* xq, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3,
+                          const void* s3, const void* w2, const void* s2, int I, const float* add, float* y, void* ws, int topk, int E, hipStream_t st)
+{
+    return ds41_moe_mx_ex(xq, xs, R, idx, rw, w1, s1, w3, s3, w2, s2, I, add, y, ws, topk, E, 0, st);
+}
+SPARK_API int ds41_moe_mx_combine_rows(void* ws, int R, int I, int topk, int E, const float* add, float* y, int r0, int nr, hipStream_t st)
+{
+    if (r0 < 0 || nr < 1 || r0 + nr > R) return 1;
+    const WsLayout l = ws_layout(R, DS41_H, I, topk, E);
+    const int* pairmap = (const int*)((char*)ws + l.pairmap);
+    const float* out = (const float*)((char*)ws + l.out);
+    const int64_t n4 = (int64_t)nr * (DS41_H / 4);
+    combine_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(out, pairmap + (int64_t)r0 * topk, add ? add + (int64_t)r0 * DS41_H : nullptr,
+                                                                 y + (int64_t)r0 * DS41_H, nr, DS41_H, topk, 0);
+    return launch_status();
+}
+SPARK_API int ds41_moe_mx_combine(void* ws, int R, int I, int topk, int E, const float* add, float* y, hipStream_t st)
+{
+    return ds41_moe_mx_combine_rows(ws, R, I, topk, E, add, y, 0, R, st);
+}
+SPARK_API int ds41_moe_mx_ws_ptrs(void* ws, int R, int I, int topk, int E, float** out, int** pairmap)
+{
+    const WsLayout l = ws_layout(R, DS41_H, I, topk, E);
+    *pairmap = (int*)((char*)ws + l.pairmap);
+    *out = (float*)((char*)ws + l.out);
+    return 0;
+}
+// reference ds41_moe.cu:266-291: xq is the act-quantized input as BF16 values; weights in the moe_pack tile layout
+// (kern.rs:718-726).  The BF16 values are re-encoded as E4M3 + UE8M0 (exactly: act_quant is idempotent) in the tail of ws.
+SPARK_API int ds41_moe(const void* xq, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3, const void* s3,
+                       const void* w2, const void* s2, int I, const float* add, float* y, void* ws, int topk, int E, hipStream_t st)
+{
+    if (R < 1 || I % 128 != 0 || E > 384 || topk < 1) return 1;
+    char* tail = (char*)ws + spark_mxfp4_moe_ws_bytes(R, DS41_H, I, topk, E, 0);
+    uint8_t* q = (uint8_t*)tail;
+    uint8_t* qs = (uint8_t*)(tail + align256((size_t)R * DS41_H));
+    const int rc = ds41_act_quant_fp8(xq, q, qs, (long long)R * DS41_H, st);
+    if (rc) return rc;
+    return moe_launch<L_PACK8>(q, qs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3, (const uint8_t*)s3, (const uint8_t*)w2,
+                               (const uint8_t*)s2, DS41_H, I, topk, E, 0, add, y, ws, 0, st);
+}

@@ -1,0 +1,337 @@
+"""Host-side mirror of the reference engine's kernel wrappers (engine-rs/src/ds41/kern.rs, src/qwen/ffi.rs,
+src/moe_own.rs): tensors in, raw device pointers + the current stream into the C ABI, a non-zero return code raises
+(the Rust wrappers `assert_eq!(rc, 0)`).  torch is used for device memory and the stream only.
+"""
+import ctypes as C
+
+import torch
+
+from . import lib as _l
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _lib():
+    return _l.load()
+
+
+def _st():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _ck(rc, name):
+    if rc != 0:
+        raise KernelError(f"{name} returned {rc}")
+
+
+def _dev(t):
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensor expected"
+    return t
+
+
+# ---------------------------------------------------------------- dequantisation surfaces
+
+def exl3_reconstruct(trellis, codebook=2):
+    """trellis int16 [Kt, Nt, 16*bits] -> inner fp16 [K, N].  reference qwen_exl3.cu qwen_exl3_reconstruct."""
+    Kt, Nt, W = trellis.shape
+    out = torch.empty(Kt * 16, Nt * 16, dtype=torch.float16, device=trellis.device)
+    _ck(_lib().spark_exl3_reconstruct(_p(_dev(trellis)), _p(out), Kt * 16, Nt * 16, W // 16, codebook, _st()), "spark_exl3_reconstruct")
+    return out
+
+
+def exl3_fold(trellis, suh, svh, codebook=2):
+    """-> W^T fp16 [N, K].  reference qwen_exl3.cu qwen_exl3_fold."""
+    Kt, Nt, W = trellis.shape
+    K, N = Kt * 16, Nt * 16
+    out = torch.empty(N, K, dtype=torch.float16, device=trellis.device)
+    _ck(_lib().spark_exl3_fold(_p(_dev(trellis)), _p(_dev(suh)), _p(_dev(svh)), K, N, W // 16, codebook, _p(out), K, _st()), "spark_exl3_fold")
+    return out
+
+
+def mxfp4_dequant(w, s):
+    N, K = w.shape[0], w.shape[1] * 2
+    out = torch.empty(N, K, dtype=torch.float32, device=w.device)
+    _ck(_lib().spark_mxfp4_dequant(_p(_dev(w)), _p(_dev(s)), _p(out), N, K, _st()), "spark_mxfp4_dequant")
+    return out
+
+
+def fp8_block_dequant(w, s, bs=128):
+    N, K = w.shape
+    out = torch.empty(N, K, dtype=torch.float32, device=w.device)
+    _ck(_lib().spark_fp8_block_dequant(_p(_dev(w)), _p(_dev(s)), _p(out), N, K, bs, _st()), "spark_fp8_block_dequant")
+    return out
+
+
+def fp8_e8m0_dequant(w, s):
+    N, K = w.shape
+    out = torch.empty(N, K, dtype=torch.float32, device=w.device)
+    _ck(_lib().spark_fp8_e8m0_dequant(_p(_dev(w)), _p(_dev(s)), _p(out), N, K, _st()), "spark_fp8_e8m0_dequant")
+    return out
+
+
+# ---------------------------------------------------------------- act_quant (reference kern.rs act_quant / act_quant_fp8)
+
+def act_quant(x):
+    """bf16 -> quantize-dequantize bf16 (UE8M0 per 32)."""
+    out = torch.empty_like(x)
+    _ck(_lib().ds41_act_quant32(_p(_dev(x)), _p(out), x.numel(), _st()), "ds41_act_quant32")
+    return out
+
+
+def act_quant_fp8(x):
+    """bf16 [R, K] -> (q uint8 [R, K], s uint8 [R, K/32])."""
+    x = _dev(x)
+    q = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    s = torch.empty(*x.shape[:-1], x.shape[-1] // 32, dtype=torch.uint8, device=x.device)
+    _ck(_lib().ds41_act_quant_fp8(_p(x), _p(q), _p(s), x.numel(), _st()), "ds41_act_quant_fp8")
+    return q, s
+
+
+def swiglu_quant(gu, lim):
+    T, I2 = gu.shape
+    out = torch.empty(T, I2 // 2, dtype=torch.bfloat16, device=gu.device)
+    _ck(_lib().ds41_swiglu_quant(_p(_dev(gu)), _p(out), T, I2 // 2, float(lim), _st()), "ds41_swiglu_quant")
+    return out
+
+
+# ---------------------------------------------------------------- routers
+
+def softmax_route(logits, topk):
+    """reference qwen/ffi.rs moe_route: logits f32 [R, E] -> (idx int32 [R, topk], w f32)."""
+    R, E = logits.shape
+    idx = torch.empty(R, topk, dtype=torch.int32, device=logits.device)
+    w = torch.empty(R, topk, dtype=torch.float32, device=logits.device)
+    _ck(_lib().spark_softmax_route(_p(_dev(logits)), logits.stride(0), R, E, topk, _p(idx), _p(w), _st()), "spark_softmax_route")
+    return idx, w
+
+
+def qwen_moe_route(logits):
+    R = logits.shape[0]
+    idx = torch.empty(R, 10, dtype=torch.int32, device=logits.device)
+    w = torch.empty(R, 10, dtype=torch.float32, device=logits.device)
+    _ck(_lib().qwen_moe_route_ld(_p(logits), logits.stride(0), R, _p(idx), _p(w), _st()), "qwen_moe_route_ld")
+    return idx, w
+
+
+def route(logits, bias, k, scale):
+    """reference kern.rs route (ds41_route): -> (idx int64 [T, k], w f32 [T, k])."""
+    T, E = logits.shape
+    idx = torch.empty(T, k, dtype=torch.int64, device=logits.device)
+    w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    _ck(_lib().ds41_route(_p(_dev(logits)), _p(_dev(bias)), _p(idx), _p(w), T, E, k, float(scale), _st()), "ds41_route")
+    return idx, w
+
+
+def sigmoid_route(logits, bias, k, scaling):
+    T, E = logits.shape
+    idx = torch.empty(T, k, dtype=torch.int64, device=logits.device)
+    w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    _ck(_lib().spark_sigmoid_route(_p(_dev(logits)), _p(_dev(bias)), _p(idx), _p(w), T, E, k, float(scaling), _st()), "spark_sigmoid_route")
+    return idx, w
+
+
+def glm_router_fused(h, w, bias, scaling):
+    """reference moe.rs route() -> rs_router_fused -> glm53_router_fused_cuda: h f32 [rows, k], w f32|bf16 [E, k]."""
+    rows, k = h.shape
+    E = w.shape[0]
+    partial = torch.empty(rows, E, 2, dtype=torch.float32, device=h.device)
+    ids = torch.empty(rows, 8, dtype=torch.int64, device=h.device)
+    wt = torch.empty(rows, 8, dtype=torch.float32, device=h.device)
+    _ck(_lib().glm53_router_fused_cuda(_p(_dev(h)), _p(_dev(w)), int(w.dtype == torch.bfloat16), _p(_dev(bias)), _p(partial), _p(ids), _p(wt),
+                                       rows, E, k, float(scaling), _st()), "glm53_router_fused_cuda")
+    return ids, wt
+
+
+# ---------------------------------------------------------------- dense GEMVs (reference kern.rs mxfp4_gemv / fp8_gemv)
+
+def mxfp4_gemv(x, w, s):
+    m, k = x.shape
+    n = w.shape[0]
+    y = torch.empty(m, n, dtype=torch.float32, device=x.device)
+    _ck(_lib().ds41_mxfp4_gemv(_p(_dev(x)), _p(_dev(w)), _p(_dev(s)), _p(y), m, n, k, _st()), "ds41_mxfp4_gemv")
+    return y
+
+
+def fp8_gemv(x, w, s):
+    m, k = x.shape
+    n = w.shape[0]
+    y = torch.empty(m, n, dtype=torch.float32, device=x.device)
+    _ck(_lib().ds41_fp8_gemv(_p(_dev(x)), _p(_dev(w)), _p(_dev(s)), _p(y), m, n, k, _st()), "ds41_fp8_gemv")
+    return y
+
+
+def fp8_block128_gemv(x, w, scales, y=None):
+    m, k = x.shape
+    n = w.shape[0]
+    if y is None:
+        y = torch.empty(m, n, dtype=torch.float32, device=x.device)
+    _ck(_lib().spark_fp8_block128_gemv(_p(_dev(x)), _p(_dev(w)), _p(_dev(scales)), _p(y), m, n, k, _st()), "spark_fp8_block128_gemv")
+    return y
+
+
+def bf16_gemv(x, w):
+    m, k = x.shape
+    n = w.shape[0]
+    y = torch.empty(m, n, dtype=torch.float32, device=x.device)
+    _ck(_lib().ds41_bf16_gemv(_p(_dev(x)), _p(_dev(w)), _p(y), m, n, k, _st()), "ds41_bf16_gemv")
+    return y
+
+
+# ---------------------------------------------------------------- MXFP4 MoE
+
+class Mxfp4Experts:
+    """Stacked expert weights of one layer resident on the GPU (E routed + n_shared shared experts), packed once into
+    the matrix-unit record layout, like the reference packs at load (kern.rs moe_pack / moe_pack_mx)."""
+
+    def __init__(self, w1, s1, w3, s3, w2, s2, n_shared=0, keep_natural=False):
+        ET, I, H2 = w1.shape
+        self.E, self.n_shared, self.I, self.H = ET - n_shared, n_shared, I, H2 * 2
+        self.packed = [self._pack(w1, s1), self._pack(w3, s3), self._pack(w2, s2)]
+        self.natural = (w1, s1, w3, s3, w2, s2) if keep_natural else None
+
+    @staticmethod
+    def _pack(w, s):
+        rows, K = w.shape[0] * w.shape[1], w.shape[2] * 2
+        nbytes = _lib().spark_mxfp4_packed_bytes(rows, K)
+        if nbytes == 0:
+            raise KernelError(f"spark_mxfp4_packed_bytes: unsupported shape rows {rows} K {K}")
+        out = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+        _ck(_lib().spark_mxfp4_prepack(_p(_dev(w)), _p(_dev(s)), _p(out), rows, K, _st()), "spark_mxfp4_prepack")
+        return out
+
+
+def mxfp4_moe_ws(R, ex, topk):
+    n = _lib().spark_mxfp4_moe_ws_bytes(R, ex.H, ex.I, topk, ex.E, ex.n_shared)
+    if n == 0:
+        raise KernelError("spark_mxfp4_moe_ws_bytes: unsupported shape")
+    return n
+
+
+def mxfp4_moe(x, idx, rw, ex, add=None, y=None, ws=None, scratch=None, natural=False):
+    """x bf16 [R, H] -> y f32 [R, H] (reference kern.rs moe_mx: act_quant_fp8 + ds41_moe_mx, with runtime sizes and the
+    shared experts folded in)."""
+    R, H = x.shape
+    topk = idx.shape[1]
+    dev = x.device
+    if y is None:
+        y = torch.empty(R, H, dtype=torch.float32, device=dev)
+    if ws is None:
+        ws = torch.empty(mxfp4_moe_ws(R, ex, topk), dtype=torch.uint8, device=dev)
+    if scratch is None:
+        scratch = (torch.empty(R, H, dtype=torch.uint8, device=dev), torch.empty(R, H // 32, dtype=torch.uint8, device=dev))
+    if natural:
+        w1, s1, w3, s3, w2, s2 = ex.natural
+        layout = 1
+    else:
+        (w1, w3, w2), (s1, s3, s2), layout = ex.packed, (None, None, None), 0
+    _ck(_lib().spark_mxfp4_moe(_p(_dev(x)), _p(scratch[0]), _p(scratch[1]), R, _p(_dev(idx)), _p(_dev(rw)), _p(w1), _p(s1), _p(w3), _p(s3), _p(w2), _p(s2),
+                               layout, H, ex.I, topk, ex.E, ex.n_shared, _p(add), _p(y), _p(ws), _st()), "spark_mxfp4_moe")
+    return y
+
+
+# reference tile layouts (kern.rs:718-734), restated with tensor view/permute exactly as the Rust does
+def moe_pack(w, s):
+    e, rows, kb = w.shape
+    steps = kb // 64
+    wp = w.view(e * rows // 8, 8, steps, 4, 16).permute(0, 2, 1, 3, 4).contiguous()
+    sp = s.view(e * rows // 8, 8, steps, 4).permute(0, 2, 1, 3).contiguous()
+    return wp.view(e, rows, kb), sp.view(e, rows, kb // 16)
+
+
+def moe_pack_mx(wp):
+    e, rows, kb = wp.shape
+    steps = kb // 64
+    return wp.view(e * rows // 8, steps, 8, 4, 4, 4).permute(0, 1, 2, 4, 3, 5).contiguous().view(e, rows, kb)
+
+
+def ds41_moe_mx(xq, xs, idx, rw, w, I, add=None, skip_combine=False, ws=None):
+    """reference kern.rs moe_mx_par / ds41_moe_mx_ex: hidden 5120, weights w = (w1, s1, w3, s3, w2, s2) in the mx tile layout."""
+    R = xq.shape[0]
+    topk, E = idx.shape[1], w[0].shape[0]
+    y = torch.empty(R, 5120, dtype=torch.float32, device=xq.device)
+    if ws is None:
+        ws = torch.empty(_lib().ds41_moe_mx_ws_bytes(R, I, topk, E), dtype=torch.uint8, device=xq.device)
+    _ck(_lib().ds41_moe_mx_ex(_p(_dev(xq)), _p(_dev(xs)), R, _p(_dev(idx)), _p(_dev(rw)), *[_p(_dev(t)) for t in w], I, _p(add), _p(y), _p(ws), topk, E,
+                              int(skip_combine), _st()), "ds41_moe_mx_ex")
+    return y, ws
+
+
+def ds41_moe(xq_bf16, idx, rw, w, I, add=None):
+    """reference kern.rs moe (ds41_moe): weights in the moe_pack tile layout, xq the act-quantized input as bf16."""
+    R = xq_bf16.shape[0]
+    topk, E = idx.shape[1], w[0].shape[0]
+    y = torch.empty(R, 5120, dtype=torch.float32, device=xq_bf16.device)
+    ws = torch.empty(_lib().ds41_moe_ws_bytes(R, I, topk, E), dtype=torch.uint8, device=xq_bf16.device)
+    _ck(_lib().ds41_moe(_p(_dev(xq_bf16)), R, _p(_dev(idx)), _p(_dev(rw)), *[_p(_dev(t)) for t in w], I, _p(add), _p(y), _p(ws), topk, E, _st()), "ds41_moe")
+    return y
+
+
+# ---------------------------------------------------------------- EXL3 MoE (reference reference/qwen38/kern.py ExpertTable / moe_routed,
+# engine-rs/src/qwen/ffi.rs moe_experts, src/moe_own.rs run_into)
+
+class ExpertTable:
+    """All experts of one layer resident on the GPU + the [9][E] device-pointer table (gate_tr, up_tr, down_tr,
+    gate_suh, up_suh, down_suh, gate_svh, up_svh, down_svh)."""
+
+    def __init__(self, experts, E, device="cuda:0"):
+        """experts: dict e -> 9 device tensors (or stacked tensors per slot, see from_stacked).  Missing experts get null pointers."""
+        self.E = E
+        self.keep = experts
+        rows = [[0] * E for _ in range(9)]
+        for e, ts in experts.items():
+            for slot, t in enumerate(ts):
+                assert t.is_cuda and t.is_contiguous()
+                rows[slot][e] = t.data_ptr()
+        self.tab = torch.tensor(rows, dtype=torch.int64, device=device).contiguous()
+
+    @classmethod
+    def from_stacked(cls, stacked, device="cuda:0"):
+        """stacked: 9 tensors [E, ...] (one per table slot)."""
+        E = stacked[0].shape[0]
+        return cls({e: [s[e] for s in stacked] for e in range(E)}, E, device)
+
+
+_XT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def exl3_moe_ws(R, H, I, E, topk):
+    n = _lib().spark_exl3_moe_ws_bytes(R, H, I, E, topk)
+    if n == 0:
+        raise KernelError("spark_exl3_moe_ws_bytes: unsupported shape")
+    return n
+
+
+def exl3_moe(x, idx, w, table, H, I, codebook=2, act=0, add=None, out=None, ws=None):
+    """x [R, H] f32 | f16 | bf16, idx int32 | int64 [R, topk], w f32 | f16 [R, topk] -> out f32 [R, H]."""
+    R, topk = idx.shape
+    if out is None:
+        out = torch.empty(R, H, dtype=torch.float32, device=x.device)
+    if ws is None:
+        ws = torch.empty(exl3_moe_ws(R, H, I, table.E, topk), dtype=torch.uint8, device=x.device)
+    _ck(_lib().spark_exl3_moe(_p(x), _XT[x.dtype], x.stride(0), R, _p(_dev(idx)), int(idx.dtype == torch.int64), _p(_dev(w)), int(w.dtype == torch.float16),
+                              _p(table.tab), _p(add), _p(out), _p(ws), H, I, table.E, topk, codebook, act, _st()), "spark_exl3_moe")
+    return out
+
+
+def qwen_moe_experts(x, idx, w, table, add=None, S=4):
+    """reference qwen/ffi.rs moe_experts: x f32 [R, 2560], 512 experts, top-10."""
+    R = x.shape[0]
+    ws = torch.empty(_lib().qwen_moe_ws_bytes(R, S), dtype=torch.uint8, device=x.device)
+    out = torch.empty(R, 2560, dtype=torch.float32, device=x.device)
+    _ck(_lib().qwen_moe_experts(_p(x), x.stride(0), R, _p(_dev(idx)), _p(_dev(w)), _p(table.tab), _p(add), _p(out), _p(ws), S, _st()), "qwen_moe_experts")
+    return out
+
+
+def glm_moe_experts(x, idx, w, table, add=None, S=2, kmask=1 << 4):
+    """reference moe_own.rs run_into: x f16 [R, 4096], idx int64 / w f16 [R, 8], 288 experts, mcg codebook."""
+    R = x.shape[0]
+    ws = torch.empty(_lib().glm_moe_ws_bytes(R, S), dtype=torch.uint8, device=x.device)
+    out = torch.empty(R, 4096, dtype=torch.float32, device=x.device)
+    _ck(_lib().glm_moe_experts(_p(x), x.stride(0), R, _p(_dev(idx)), _p(_dev(w)), _p(table.tab), _p(add), _p(out), _p(ws), S, None, kmask, _st()), "glm_moe_experts")
+    return out

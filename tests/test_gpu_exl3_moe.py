@@ -1,0 +1,102 @@
+"""GPU parity of the routed EXL3 experts against the CPU oracle (dequantise to FP32 + FP32 matmul, the reference's
+CPU path).  Tolerance: rel-L2 <= 1e-3 on the FP32 output (reference test_kern_moe.py:24, kern.rs:2206)."""
+import numpy as np
+import pytest
+import torch
+
+from spark_engine_amd import synth
+from tests.gpu_util import DEV, dev, dev_bf16, dev_f16, host, rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from spark_engine_amd import ops
+    return ops
+
+
+def _layer(g, E_used, H, I):
+    return {e: synth.exl3_expert(g, H, I) for e in E_used}
+
+
+def _to_dev(experts):
+    out = {}
+    for e, t in experts.items():
+        out[e] = [dev(t[0]), dev(t[1]), dev(t[2])] + [dev_f16(a) for a in t[3:]]
+    return out
+
+
+@pytest.mark.parametrize("cbk,act", [(2, 0), (1, 1)])
+@pytest.mark.parametrize("R,H,I,E,topk", [(1, 256, 128, 4, 2), (1, 2048, 512, 512, 10), (4, 2048, 512, 512, 10), (3, 512, 384, 16, 4)])
+def test_exl3_moe_vs_oracle(ops, oracle, cbk, act, R, H, I, E, topk):
+    g = synth.rng(400 + R + H + cbk)
+    logits = g.standard_normal((R, E)).astype(np.float32)
+    idx, w = oracle.qwen_route(logits, topk)
+    used = sorted(set(idx.ravel().tolist()))
+    experts = _layer(g, used, H, I)
+    xb = synth.randn_bf16(g, (R, H))
+    add = g.standard_normal((R, H)).astype(np.float32)
+    ref = oracle.exl3_moe(synth.bf16_to_f32(xb), idx, w, experts, E, H, I, 4, cbk, act, add)
+    table = ops.ExpertTable(_to_dev(experts), E)
+    out = host(ops.exl3_moe(dev_bf16(xb), dev(idx), dev(w), table, H, I, cbk, act, add=dev(add)))
+    assert rel_l2(out, ref) <= TOL, rel_l2(out, ref)
+    out2 = host(ops.exl3_moe(dev_bf16(xb), dev(idx), dev(w), table, H, I, cbk, act, add=dev(add)))
+    assert np.array_equal(out, out2)                                 # deterministic (reference test_kern_moe.py:23-24)
+
+
+def test_exl3_moe_shared_experts_and_row_invariance(ops, oracle):
+    g = synth.rng(410)
+    R, H, I, E, topk = 5, 512, 256, 6, 3
+    experts = _layer(g, range(E), H, I)
+    idx = np.array([[0, 1, 2], [1, 0, 5], [0, 4, 1], [2, 1, 0], [3, 0, 1]], np.int32)    # experts 0 and 1 take 5 rows
+    w = g.uniform(0.1, 1, (R, topk)).astype(np.float32)
+    x = g.standard_normal((R, H)).astype(np.float32)
+    table = ops.ExpertTable(_to_dev(experts), E)
+    out = host(ops.exl3_moe(dev(x), dev(idx), dev(w), table, H, I))
+    ref = oracle.exl3_moe(x, idx, w, experts, E, H, I, 4, 2, 0)
+    assert rel_l2(out, ref) <= TOL
+    for r in range(R):
+        o1 = host(ops.exl3_moe(dev(x[r:r + 1]), dev(idx[r:r + 1]), dev(w[r:r + 1]), table, H, I))
+        assert np.array_equal(o1[0], out[r])                          # a row's bits do not depend on the batch
+
+
+def test_exl3_moe_sixteen_rows_one_expert(ops, oracle):
+    g = synth.rng(411)
+    R, H, I, E, topk = 16, 256, 128, 3, 1
+    experts = _layer(g, range(E), H, I)
+    idx = np.full((R, 1), 2, np.int32)
+    w = g.uniform(0.5, 1, (R, 1)).astype(np.float32)
+    x = g.standard_normal((R, H)).astype(np.float32)
+    table = ops.ExpertTable(_to_dev(experts), E)
+    out = host(ops.exl3_moe(dev(x), dev(idx), dev(w), table, H, I))
+    assert rel_l2(out, oracle.exl3_moe(x, idx, w, experts, E, H, I, 4, 2, 0)) <= TOL
+
+
+def test_reference_symbols_qwen_and_glm(ops, oracle):
+    # the reference's fixed-size entry points: Qwen 512 x top-10, H 2560, I 640, f32 in; GLM 288 x top-8, H 4096, I 1024, f16 in
+    g = synth.rng(412)
+    R = 2
+    logits = g.standard_normal((R, 512)).astype(np.float32)
+    idx, w = ops.qwen_moe_route(dev(logits))
+    idx_h, w_h = host(idx), host(w)
+    experts = _layer(g, sorted(set(idx_h.ravel().tolist())), 2560, 640)
+    x = (g.standard_normal((R, 2560)) * 0.3).astype(np.float32)
+    table = ops.ExpertTable(_to_dev(experts), 512)
+    out = host(ops.qwen_moe_experts(dev(x), idx, w, table))
+    assert rel_l2(out, oracle.exl3_moe(x, idx_h, w_h, experts, 512, 2560, 640, 4, 2, 0)) <= TOL
+    idx8 = np.stack([g.permutation(288)[:8] for _ in range(R)]).astype(np.int64)
+    w8 = (g.uniform(0, 1, (R, 8)) + 0.1).astype(np.float16)
+    ex2 = _layer(g, sorted(set(idx8.ravel().tolist())), 4096, 1024)
+    x16 = g.standard_normal((R, 4096)).astype(np.float16)
+    t2 = ops.ExpertTable(_to_dev(ex2), 288)
+    out = host(ops.glm_moe_experts(dev_f16(x16.view(np.uint16)), dev(idx8), dev_f16(w8.view(np.uint16)), t2))
+    ref = oracle.exl3_moe(x16.astype(np.float32), idx8.astype(np.int32), w8.astype(np.float32), ex2, 288, 4096, 1024, 4, 1, 1)
+    assert rel_l2(out, ref) <= TOL
+
+
+def test_exl3_moe_rejects_bad_shapes(ops):
+    x = torch.zeros(1, 200, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.exl3_moe_ws(1, 200, 128, 4, 2)                            # H not a multiple of 128

@@ -1,0 +1,172 @@
+"""GPU parity: dequantisation surfaces (bit-exact), act_quant (bit-exact), routers (exact indices), dense GEMVs.
+Every call goes through the C ABI of libspark_shim_hip.so."""
+import numpy as np
+import pytest
+import torch
+
+from spark_engine_amd import synth
+from tests.gpu_util import DEV, dev, dev_bf16, dev_f16, host, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from spark_engine_amd import ops
+    return ops
+
+
+@pytest.mark.parametrize("cbk", [2, 1])
+@pytest.mark.parametrize("bits", [4, 3, 5, 6])
+def test_exl3_reconstruct_bit_exact(ops, oracle, cbk, bits):
+    g = synth.rng(100 + bits)
+    tr = g.integers(-32768, 32768, (24, 9, 16 * bits), dtype=np.int16)
+    got = host(ops.exl3_reconstruct(dev(tr), cbk))
+    assert np.array_equal(got, oracle.decode_inner(tr, cbk))
+
+
+def test_exl3_reconstruct_all_codebook_states(ops, oracle):
+    # a 4-bit tile stream visits the states of its nibble 4-grams: cover the whole codebook with a De Bruijn-free trick,
+    # 4096 tiles of random bits and compare the multiset of decoded values against the tables
+    g = synth.rng(7)
+    tr = g.integers(-32768, 32768, (64, 64, 64), dtype=np.int16)
+    for cbk in (1, 2):
+        assert np.array_equal(host(ops.exl3_reconstruct(dev(tr), cbk)), oracle.decode_inner(tr, cbk))
+
+
+@pytest.mark.parametrize("cbk,bits", [(2, 4), (1, 4), (2, 5)])
+def test_exl3_fold_bit_exact(ops, oracle, cbk, bits):
+    g = synth.rng(110 + bits + cbk)
+    K, N = 256, 384
+    tr, suh, svh = synth.exl3_matrix(g, K, N, bits)
+    got = host(ops.exl3_fold(dev(tr), dev_f16(suh), dev_f16(svh), cbk))
+    assert np.array_equal(got, oracle.fold(tr, suh, svh, cbk))
+
+
+def test_mxfp4_dequant_bit_exact(ops, oracle):
+    g = synth.rng(120)
+    w, s = synth.mxfp4_matrix(g, 96, 512, 1, 250)
+    assert np.array_equal(host(ops.mxfp4_dequant(dev(w), dev(s))), oracle.mxfp4_dequant(w, s))
+    # every byte value under one scale
+    w = np.tile(np.arange(256, dtype=np.uint8), (4, 1)).reshape(4, 256)[:, :64].copy(); w = np.arange(256, dtype=np.uint8).reshape(16, 16)
+    s = np.full((16, 1), 125, np.uint8)
+    assert np.array_equal(host(ops.mxfp4_dequant(dev(w), dev(s))), oracle.mxfp4_dequant(w, s))
+
+
+def test_fp8_dequant_bit_exact(ops, oracle):
+    g = synth.rng(121)
+    w = g.integers(0, 256, (256, 384), dtype=np.uint8)
+    w[(w & 0x7f) == 0x7f] = 0x12
+    w[0, :256] = np.arange(256, dtype=np.uint8); w[0, 0x7f] = 0; w[0, 0xff] = 0   # every finite code
+    s = np.exp(g.uniform(np.log(1e-3), np.log(1e-1), (2, 3))).astype(np.float32)
+    assert np.array_equal(host(ops.fp8_block_dequant(dev(w), dev(s), 128)), oracle.fp8_block_dequant(w, s, 128))
+    s8 = g.integers(100, 135, (8, 12), dtype=np.uint8)
+    assert np.array_equal(host(ops.fp8_e8m0_dequant(dev(w), dev(s8))), oracle.fp8_e8m0_dequant(w, s8))
+
+
+def test_act_quant_bit_exact(ops, oracle):
+    g = synth.rng(122)
+    x = g.standard_normal((512, 64), np.float32) * (10.0 ** g.uniform(-6, 3, (512, 1))).astype(np.float32)
+    x[:8] = 0
+    x[8:72, 0] = (448.0 * 2.0 ** np.arange(-32, 32)).astype(np.float32)
+    xb = synth.bf16_bits(x)
+    q, s = ops.act_quant_fp8(dev_bf16(xb))
+    qo, so = oracle.act_quant_fp8(xb)
+    assert np.array_equal(host(s), so)
+    qh = host(q)
+    z = (qo & 0x7f) == 0
+    assert np.array_equal(qh[~z], qo[~z]) and np.all((qh[z] & 0x7f) == 0)
+    d = host(ops.act_quant(dev_bf16(xb)))
+    assert np.array_equal(synth.bf16_to_f32(d), synth.bf16_to_f32(oracle.act_quant32(xb)))
+
+
+def test_act_quant_every_bf16_value(ops, oracle):
+    # all 65536 bf16 patterns (finite ones) in blocks that share a large amax, and alone in a block
+    bits = np.arange(65536, dtype=np.uint16)
+    f = synth.bf16_to_f32(bits)
+    ok = np.isfinite(f) & (np.abs(f) < 1e30)
+    bits = bits[ok]
+    pad = (-len(bits)) % 32
+    bits = np.concatenate([bits, np.zeros(pad, np.uint16)]).reshape(-1, 32)
+    q, s = ops.act_quant_fp8(dev_bf16(bits))
+    qo, so = oracle.act_quant_fp8(bits)
+    assert np.array_equal(host(s), so)
+    qh = host(q); z = (qo & 0x7f) == 0
+    assert np.array_equal(qh[~z], qo[~z]) and np.all((qh[z] & 0x7f) == 0)
+
+
+def test_routers_exact_indices(ops, oracle):
+    g = synth.rng(130)
+    lq = g.standard_normal((5, 512)).astype(np.float32)
+    idx, w = ops.qwen_moe_route(dev(lq))
+    io, wo = oracle.qwen_route(lq, 10)
+    assert np.array_equal(host(idx), io) and np.allclose(host(w), wo, rtol=1e-5)
+    idx, w = ops.softmax_route(dev(lq[:, :300].copy()), 6)
+    io, wo = oracle.qwen_route(lq[:, :300].copy(), 6)
+    assert np.array_equal(host(idx), io) and np.allclose(host(w), wo, rtol=1e-5)
+    ld = g.standard_normal((7, 384)).astype(np.float32) * 3
+    ld[0, 3] = 25.0
+    bias = (g.standard_normal(384) * 0.1).astype(np.float32)
+    idx, w = ops.route(dev(ld), dev(bias), 6, 1.5)
+    io, wo = oracle.ds41_route(ld, bias, 6, 1.5)
+    assert np.array_equal(host(idx), io) and np.allclose(host(w), wo, rtol=2e-6)
+    idx, w = ops.sigmoid_route(dev(ld[:, :288].copy()), dev(bias[:288].copy()), 8, 2.5)
+    io, wo = oracle.glm_route(ld[:, :288].copy(), bias[:288].copy(), 8, 2.5)
+    assert np.array_equal(host(idx), io) and np.allclose(host(w), wo, rtol=2e-6)
+    # ties go to the lower expert id
+    t = np.zeros((1, 512), np.float32); t[0, [400, 17, 300]] = 1.0
+    idx, _ = ops.qwen_moe_route(dev(t))
+    assert host(idx)[0].tolist() == [17, 300, 400, 0, 1, 2, 3, 4, 5, 6]
+    idx, _ = ops.route(dev(np.zeros((2, 384), np.float32)), dev(np.zeros(384, np.float32)), 6, 1.0)
+    assert host(idx).tolist() == [[0, 1, 2, 3, 4, 5]] * 2
+
+
+def test_glm_router_fused(ops, oracle):
+    g = synth.rng(131)
+    h = g.standard_normal((3, 1024)).astype(np.float32)
+    wg = (g.standard_normal((288, 1024)) * 0.05).astype(np.float32)
+    bias = (g.standard_normal(288) * 0.1).astype(np.float32)
+    ids, wt = ops.glm_router_fused(dev(h), dev(wg), dev(bias), 2.5)
+    logits = (h.astype(np.float64) @ wg.astype(np.float64).T).astype(np.float32)
+    io, wo = oracle.glm_route(logits, bias, 8, 2.5)
+    assert np.array_equal(host(ids), io) and np.allclose(host(wt), wo, rtol=1e-4)
+
+
+@pytest.mark.parametrize("m", [1, 2, 4, 7])
+def test_mxfp4_gemv(ops, oracle, m):
+    # config 1 shape at m = 1: W 2048 x 2048, scales 2^-8 .. 2^0
+    g = synth.rng(0)
+    n, k = (2048, 2048) if m == 1 else (200, 1024)
+    w, s = synth.mxfp4_matrix(g, n, k, 119)
+    x = synth.randn_bf16(g, (m, k))
+    y = host(ops.mxfp4_gemv(dev_bf16(x), dev(w), dev(s)))
+    ref = oracle.mxfp4_gemv(x, w, s)
+    assert np.abs(y - ref).max() / np.abs(ref).max() < 1e-5         # the reference's own GEMV threshold (kern.rs:1863-1867)
+    assert rel_l2(y, ref) < 1e-5
+
+
+@pytest.mark.parametrize("m", [1, 4])
+def test_fp8_gemvs(ops, oracle, m):
+    g = synth.rng(140 + m)
+    n, k = 384, 1024
+    w8, s = synth.fp8_block_matrix(g, n, k)
+    x = synth.randn_bf16(g, (m, k))
+    y = host(ops.fp8_block128_gemv(dev_bf16(x), dev(w8), dev(s)))
+    ref = oracle.fp8_block_gemv(x, w8, s)
+    assert np.abs(y - ref).max() / np.abs(ref).max() < 1e-5 and rel_l2(y, ref) < 1e-5
+    s8 = g.integers(110, 128, (n // 32, k // 32), dtype=np.uint8)
+    y = host(ops.fp8_gemv(dev_bf16(x), dev(w8), dev(s8)))
+    ref = oracle.fp8_e8m0_gemv(x, w8, s8)
+    assert np.abs(y - ref).max() / np.abs(ref).max() < 1e-5 and rel_l2(y, ref) < 1e-5
+    wb = synth.randn_bf16(g, (n, k))
+    y = host(ops.bf16_gemv(dev_bf16(x), dev_bf16(wb)))
+    ref = synth.bf16_to_f32(x).astype(np.float64) @ synth.bf16_to_f32(wb).astype(np.float64).T
+    assert rel_l2(y, ref) < 1e-5
+
+
+def test_gemv_rejects_bad_shapes(ops):
+    x = torch.zeros(9, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(8, 32, dtype=torch.uint8, device=DEV)
+    s = torch.zeros(8, 2, dtype=torch.uint8, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.mxfp4_gemv(x, w, s)                                       # m > 8 -> return code 1 (reference ds41.cu:230)

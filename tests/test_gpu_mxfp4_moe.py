@@ -1,0 +1,103 @@
+"""GPU parity of the routed MXFP4 experts against the CPU oracle (dequantise + FP32 matmul with the reference's
+roundings).  Tolerance: rel-L2 <= 1e-3 on the FP32 output (reference kern.rs:2206-2208)."""
+import numpy as np
+import pytest
+import torch
+
+from spark_engine_amd import synth
+from tests.gpu_util import DEV, dev, dev_bf16, host, rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from spark_engine_amd import ops
+    return ops
+
+
+def _case(g, R, H, I, E, topk, n_shared, smin=117):
+    ws = synth.mxfp4_experts(g, E + n_shared, H, I, smin)
+    x = synth.randn_bf16(g, (R, H))
+    idx = np.stack([g.permutation(E)[:topk] for _ in range(R)]).astype(np.int64)
+    rw = g.uniform(0.1, 1.0, (R, topk)).astype(np.float32)
+    rw = (rw / rw.sum(-1, keepdims=True) * 1.5).astype(np.float32)
+    return ws, x, idx, rw
+
+
+@pytest.mark.parametrize("R,H,I,E,topk,ns", [(1, 512, 256, 8, 2, 0), (1, 1024, 512, 12, 6, 1), (4, 512, 384, 6, 3, 1), (3, 640, 128, 5, 2, 2)])
+def test_moe_small_vs_oracle(ops, oracle, R, H, I, E, topk, ns):
+    g = synth.rng(200 + R + H)
+    ws, x, idx, rw = _case(g, R, H, I, E, topk, ns)
+    add = g.standard_normal((R, H)).astype(np.float32)
+    ex = ops.Mxfp4Experts(*[dev(a) for a in ws], n_shared=ns, keep_natural=True)
+    ref = oracle.mxfp4_moe(x, idx, rw, *ws, n_shared=ns, add=add)
+    y = host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex, add=dev(add)))
+    assert rel_l2(y, ref) <= TOL, rel_l2(y, ref)
+    y2 = host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex, add=dev(add), natural=True))
+    assert np.array_equal(y, y2)                                     # the record layout changes bytes in memory, not results
+    y3 = host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex, add=dev(add)))
+    assert np.array_equal(y, y3)                                     # deterministic
+
+
+def test_moe_rows_sharing_experts_and_row_invariance(ops, oracle):
+    g = synth.rng(210)
+    R, H, I, E, topk = 4, 512, 256, 4, 2
+    ws, x, idx, rw = _case(g, R, H, I, E, topk, 0)
+    idx[:] = [[0, 1], [1, 0], [0, 3], [1, 2]]                        # experts shared by several rows
+    ex = ops.Mxfp4Experts(*[dev(a) for a in ws])
+    y = host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex))
+    assert rel_l2(y, oracle.mxfp4_moe(x, idx, rw, *ws)) <= TOL
+    for r in range(R):                                                # a row's bits do not depend on the other rows
+        yr = host(ops.mxfp4_moe(dev_bf16(x[r:r + 1]), dev(idx[r:r + 1]), dev(rw[r:r + 1]), ex))
+        assert np.array_equal(yr[0], y[r])
+
+
+def test_moe_zero_codes_give_add(ops):
+    g = synth.rng(211)
+    R, H, I, E, topk = 2, 512, 256, 3, 2
+    ws, x, idx, rw = _case(g, R, H, I, E, topk, 0)
+    ws = [np.zeros_like(a) if i % 2 == 0 else a for i, a in enumerate(ws)]
+    add = g.standard_normal((R, H)).astype(np.float32)
+    ex = ops.Mxfp4Experts(*[dev(a) for a in ws])
+    assert np.array_equal(host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex, add=dev(add))), add)
+
+
+def test_moe_many_rows_multi_column_groups(ops, oracle):
+    # more than 16 rows on one expert: several MFMA column groups per item, items of 64 rows
+    g = synth.rng(212)
+    R, H, I, E, topk = 70, 1024, 512, 3, 2
+    ws, x, idx, rw = _case(g, R, H, I, E, topk, 0)
+    ex = ops.Mxfp4Experts(*[dev(a) for a in ws])
+    y = host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex))
+    assert rel_l2(y, oracle.mxfp4_moe(x, idx, rw, *ws)) <= TOL
+
+
+def test_ds41_reference_symbols_tile_layouts(ops, oracle):
+    # the reference's own entry points: hidden 5120, weights repacked as kern.rs moe_pack / moe_pack_mx do
+    g = synth.rng(213)
+    R, H, I, E, topk = 2, 5120, 128, 4, 2
+    ws, x, idx, rw = _case(g, R, H, I, E, topk, 0, smin=119)
+    add = g.standard_normal((R, H)).astype(np.float32)
+    ref = oracle.mxfp4_moe(x, idx, rw, *ws, add=add)
+    d = [dev(a) for a in ws]
+    p1, ps1 = ops.moe_pack(d[0], d[1]); p3, ps3 = ops.moe_pack(d[2], d[3]); p2, ps2 = ops.moe_pack(d[4], d[5])
+    xq, xs = ops.act_quant_fp8(dev_bf16(x))
+    y, wsb = ops.ds41_moe_mx(xq, xs, dev(idx), dev(rw), (ops.moe_pack_mx(p1), ps1, ops.moe_pack_mx(p3), ps3, ops.moe_pack_mx(p2), ps2), I, add=dev(add))
+    assert rel_l2(host(y), ref) <= TOL
+    xdq = ops.act_quant(dev_bf16(x))
+    y2 = ops.ds41_moe(xdq, dev(idx), dev(rw), (p1, ps1, p3, ps3, p2, ps2), I, add=dev(add))
+    assert np.array_equal(host(y2), host(y))                          # same operands, same instruction sequence
+    # skip_combine + combine_rows leave the same rows behind (reference ds41_mx.cu:1471-1487)
+    from spark_engine_amd import lib
+    import ctypes as C
+    L = lib.load()
+    y3, wsb3 = ops.ds41_moe_mx(xq, xs, dev(idx), dev(rw), (ops.moe_pack_mx(p1), ps1, ops.moe_pack_mx(p3), ps3, ops.moe_pack_mx(p2), ps2), I, add=dev(add), skip_combine=True)
+    y4 = torch.zeros(R, H, dtype=torch.float32, device=DEV)
+    add_d = dev(add)
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for r0 in range(R):
+        assert L.ds41_moe_mx_combine_rows(C.c_void_p(wsb3.data_ptr()), R, I, topk, E, C.c_void_p(add_d.data_ptr()), C.c_void_p(y4.data_ptr()), r0, 1, st) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(host(y4), host(y))
