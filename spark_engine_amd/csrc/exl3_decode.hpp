@@ -73,4 +73,40 @@ __device__ __forceinline__ void tile_pos(int p, int& row, int& col)
     col = (t >> 2) + ((j & 4) ? 8 : 0);
 }
 
+// ---- the wave64 GEMV tile step.  A lane holds words 4m..4m+3 of one 16x16 4-bit tile (m = lane % 8): all 16 k rows of
+// tile columns m and m + 8.  prev = word 4m-1 of the same tile (the neighbour lane's last word; lane m = 0 wraps to word 31).
+// Decodes the lane's 32 weights into 16 packed fp16 pairs: wd[j][0] = k rows (2j, 2j+1) of column m, wd[j][1] = rows
+// (2j+8, 2j+9) of column m, wd[j][2] / wd[j][3] the same rows of column m + 8.
+__device__ __forceinline__ int tile_prev_lane(int lane) { return (lane & ~7) | ((lane + 7) & 7); }
+template <int CBK>
+__device__ __forceinline__ void decode_tile32(const uint4 w, uint32_t prev, h2 (&wd)[4][4])
+{
+    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = ww[j], hi = j == 0 ? prev : ww[j - 1];
+        const uint32_t s0 = __builtin_amdgcn_alignbit(hi, lo, 28) & 0xffffu, s1 = __builtin_amdgcn_alignbit(hi, lo, 24) & 0xffffu;
+        const uint32_t s2 = __builtin_amdgcn_alignbit(hi, lo, 20) & 0xffffu, s3 = lo >> 16;
+        const uint32_t s4 = (lo >> 12) & 0xffffu, s5 = (lo >> 8) & 0xffffu, s6 = (lo >> 4) & 0xffffu, s7 = lo & 0xffffu;
+        wd[j][0] = cb_decode2<CBK>(s0, s1);
+        wd[j][1] = cb_decode2<CBK>(s2, s3);
+        wd[j][2] = cb_decode2<CBK>(s4, s5);
+        wd[j][3] = cb_decode2<CBK>(s6, s7);
+    }
+}
+// acc0 / acc1 += the k-tile's 16 activations (8 packed fp16 pairs at xp, the same for every lane) times columns m / m + 8
+__device__ __forceinline__ void dot_tile32(const h2 (&wd)[4][4], const uint32_t* xp, float& a0, float& a1)
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        h2 xa, xb;
+        const uint32_t ua = xp[j], ub = xp[j + 4];
+        __builtin_memcpy(&xa, &ua, 4); __builtin_memcpy(&xb, &ub, 4);
+        a0 = __builtin_amdgcn_fdot2(wd[j][0], xa, a0, false);
+        a0 = __builtin_amdgcn_fdot2(wd[j][1], xb, a0, false);
+        a1 = __builtin_amdgcn_fdot2(wd[j][2], xa, a1, false);
+        a1 = __builtin_amdgcn_fdot2(wd[j][3], xb, a1, false);
+    }
+}
+
 }  // namespace spk

@@ -14,7 +14,7 @@
 // the three trailing nibbles of the previous word come from the neighbour lane.  States are cut out of the 64-bit
 // window with alignbit / bfe, decoded two at a time (packed fp16 codebook arithmetic) and accumulated with
 // v_dot2_f32_f16 against the Hadamard-transformed activations, which are wave-uniform and arrive as scalar loads.
-#include "common.hpp"
+#include "moe_exl3.hpp"
 #include "exl3_decode.hpp"
 
 using namespace spk;
@@ -25,26 +25,11 @@ constexpr int EMAX = 1024;            // experts (one grouping thread each)
 constexpr int PMAX = 1024;            // routed pairs per call (decode / verify chains)
 constexpr int GV_WAVES = 4;
 
-enum XType { X_F32 = 0, X_F16 = 1, X_BF16 = 2 };
-
-struct Cfg {                          // runtime shape of one layer
-    int E, topk, H, I, cbk, act;      // act 0: silu(g) * u, 1: clamp (g <= 10, |u| <= 10) first
-    int xtype, wtype, itype;          // x: XType; route weights: 0 f32, 1 f16; indices: 0 int32, 1 int64
-};
-
-__device__ __forceinline__ float ld_x(const void* x, int xtype, int64_t i)
-{
-    if (xtype == X_F32) return ((const float*)x)[i];
-    if (xtype == X_F16) return f16_bits_to_f32(((const uint16_t*)x)[i]);
-    return bf16_to_f32(((const uint16_t*)x)[i]);
-}
-__device__ __forceinline__ int ld_idx(const void* idx, int itype, int i) { return itype ? (int)((const int64_t*)idx)[i] : ((const int*)idx)[i]; }
-__device__ __forceinline__ float ld_w(const void* w, int wtype, int i) { return wtype ? f16_bits_to_f32(((const uint16_t*)w)[i]) : ((const float*)w)[i]; }
-__device__ __forceinline__ float act_fn(int act, float a, float u)
-{
-    if (act == 1) { a = fminf(a, 10.0f); u = fminf(fmaxf(u, -10.0f), 10.0f); }
-    return a / (1.0f + __expf(-a)) * u;
-}
+typedef Exl3Cfg Cfg;
+__device__ __forceinline__ float ld_x(const void* x, int xtype, int64_t i) { return exl3_ld_x(x, xtype, i); }
+__device__ __forceinline__ int ld_idx(const void* idx, int itype, int i) { return exl3_ld_idx(idx, itype, i); }
+__device__ __forceinline__ float ld_w(const void* w, int wtype, int i) { return exl3_ld_w(w, wtype, i); }
+__device__ __forceinline__ float act_fn(int act, float a, float u) { return exl3_act(act, a, u); }
 
 // ---------------------------------------------------------------- grouping: stable counting sort of the pairs by expert
 // One workgroup, thread = expert.  Items of at most GR rows; rows ascending within an expert.
@@ -107,39 +92,15 @@ __global__ __launch_bounds__(256) void had_kernel(const void* __restrict__ x, in
 // grid (N / 128, S, T * Gmax), 4 waves.  Block (n-block nb, K slice s, matrix t, item g): rows goff[g] .. + gcnt[g] of
 // xh[t] times k-tiles [s kts, (s + 1) kts) of the expert's inner matrix, columns 128 nb .. + 127 -> part[s][t][row][N].
 // Waves interleave over the slice's k-tiles and are summed through LDS in wave order.
-__device__ __forceinline__ h2 as_h2(uint32_t v) { h2 r; __builtin_memcpy(&r, &v, 4); return r; }
-
 template <int CBK, int MR>
 __device__ __forceinline__ void tile_fma(const uint4 w, uint32_t prev, const uint32_t* __restrict__ xrow, int64_t ldx32, int rows, float (&acc)[MR][2])
 {
-    // decode this lane's 32 weights: word j holds k rows 2j, 2j+1, 2j+8, 2j+9 of column m (positions 0-3) and m+8 (4-7)
-    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
     h2 wd[4][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t lo = ww[j], hi = j == 0 ? prev : ww[j - 1];
-        const uint32_t s0 = __builtin_amdgcn_alignbit(hi, lo, 28) & 0xffffu, s1 = __builtin_amdgcn_alignbit(hi, lo, 24) & 0xffffu;
-        const uint32_t s2 = __builtin_amdgcn_alignbit(hi, lo, 20) & 0xffffu, s3 = lo >> 16;
-        const uint32_t s4 = (lo >> 12) & 0xffffu, s5 = (lo >> 8) & 0xffffu, s6 = (lo >> 4) & 0xffffu, s7 = lo & 0xffffu;
-        wd[j][0] = cb_decode2<CBK>(s0, s1);
-        wd[j][1] = cb_decode2<CBK>(s2, s3);
-        wd[j][2] = cb_decode2<CBK>(s4, s5);
-        wd[j][3] = cb_decode2<CBK>(s6, s7);
-    }
+    decode_tile32<CBK>(w, prev, wd);
 #pragma unroll
     for (int r = 0; r < MR; ++r) {
         if (r >= rows) break;
-        const uint32_t* xp = xrow + r * ldx32;       // 8 packed fp16 pairs of this k-tile (wave-uniform address)
-        float a0 = acc[r][0], a1 = acc[r][1];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const h2 xa = as_h2(xp[j]), xb = as_h2(xp[j + 4]);
-            a0 = __builtin_amdgcn_fdot2(wd[j][0], xa, a0, false);
-            a0 = __builtin_amdgcn_fdot2(wd[j][1], xb, a0, false);
-            a1 = __builtin_amdgcn_fdot2(wd[j][2], xa, a1, false);
-            a1 = __builtin_amdgcn_fdot2(wd[j][3], xb, a1, false);
-        }
-        acc[r][0] = a0; acc[r][1] = a1;
+        dot_tile32(wd, xrow + r * ldx32, acc[r][0], acc[r][1]);   // 8 packed fp16 pairs of this k-tile (wave-uniform address)
     }
 }
 
@@ -162,7 +123,7 @@ __global__ __launch_bounds__(64 * GV_WAVES) void gemv_kernel(const uint16_t* __r
     float acc[MR][2];
 #pragma unroll
     for (int r = 0; r < MR; ++r) { acc[r][0] = 0.f; acc[r][1] = 0.f; }
-    const int src = (lane & ~7) | ((lane + 7) & 7);           // lane holding the previous word of this lane's first word
+    const int src = tile_prev_lane(lane);
     // two k-tiles in flight per wave
     for (int kt = kt0 + wave; kt < kt1; kt += 2 * GV_WAVES) {
         const int ktb = kt + GV_WAVES;
@@ -289,10 +250,13 @@ void launch_gemv(const uint16_t* xh, const uint64_t* tab, int E, int slot0, cons
     else gemv_kernel<CBK, 16><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
 }
 
+// flags: bit 0 = the workspace counters are known to be zero (zeroed once, then only used by these calls);
+//        bit 1 = force the multi-kernel path
 int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
-            hipStream_t st)
+            int flags, hipStream_t st)
 {
     if (!cfg_ok(c, R)) return -1;
+    if (!(flags & 2) && exl3_fused_ok(c, R)) return exl3_fused_launch(c, x, ldx, R, idx, w, tab, add, out, ws, flags & 1, st);
     const Plan p = plan(c, R);
     char* b = (char*)ws;
     int* G = (int*)(b + p.G);
@@ -327,17 +291,26 @@ const Cfg GLM{288, 8, 4096, 1024, CB_MCG, 1, X_F16, 1, 1};
 // Runtime-sized entry (no reference counterpart symbol): x [R, H] of xtype (0 f32, 1 f16, 2 bf16), row stride ldx;
 // idx [R, topk] int32 (itype 0) or int64 (1); w [R, topk] f32 (wtype 0) or f16 (1); tab u64 [9][E]; codebook 2 = mul1,
 // 1 = mcg; act 0 = silu(g) u, 1 = clamped; add / out f32 [R, H].  4-bit trellis, R <= 64 rows.
+// flags bit 0: the workspace was zeroed by spark_exl3_moe_ws_init and only used by this entry since (saves a launch);
+// bit 1: use the multi-kernel path even where the single-launch path applies.
 SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk)
 {
     const Cfg c{E, topk, H, I, CB_MUL1, 0, 0, 0, 0};
     if (!cfg_ok(c, R)) return 0;
-    return plan(c, R).total;
+    const size_t a = plan(c, R).total, b = exl3_fused_ok(c, R) ? exl3_fused_ws_bytes(c, R) : 0;
+    return a > b ? a : b;
+}
+// zeroes the workspace once after allocation; calls made with flags bit 0 set then skip their own zeroing launch
+SPARK_API int spark_exl3_moe_ws_init(void* ws, size_t bytes, hipStream_t st)
+{
+    exl3_xcd_probe();                 // one-time placement check (synchronises; this call is made outside stream capture)
+    return (int)hipMemsetAsync(ws, 0, bytes, st);
 }
 SPARK_API int spark_exl3_moe(const void* x, int xtype, int64_t ldx, int R, const void* idx, int itype, const void* w, int wtype, const void* tab,
-                             const void* add, void* out, void* ws, int H, int I, int E, int topk, int codebook, int act, hipStream_t st)
+                             const void* add, void* out, void* ws, int H, int I, int E, int topk, int codebook, int act, int flags, hipStream_t st)
 {
     const Cfg c{E, topk, H, I, codebook, act, xtype, wtype, itype};
-    return experts(c, x, ldx, R, idx, w, tab, add, out, ws, st);
+    return experts(c, x, ldx, R, idx, w, tab, add, out, ws, flags, st);
 }
 // reference qwen_moe.cu:112-116: x f32 [R, 2560], idx i32 / w f32 [R, 10], tab u64 [9][512], out f32 [R, 2560]; S is the
 // reference's K-slice hint (the slice count is chosen from the shape here)
@@ -346,7 +319,7 @@ SPARK_API int qwen_moe_experts(const void* x, int64_t ldx, int R, const void* id
                                hipStream_t st)
 {
     (void)S;
-    return experts(QWEN, x, ldx, R, idx, w, tab, add, out, ws, st);
+    return experts(QWEN, x, ldx, R, idx, w, tab, add, out, ws, 0, st);
 }
 // reference glm_moe.cu:6-24: x f16 [R, 4096], idx i64 / w f16 [R, 8], tab u64 [10|11][288] (rows 0-8 as above), mcg codebook,
 // clamped SwiGLU.  suh0 (shared gate/up input scales) is a prefill shortcut and is not needed; kmask must be 1 << 4.
@@ -356,5 +329,5 @@ SPARK_API int glm_moe_experts(const void* x, int64_t ldx, int R, const void* idx
 {
     (void)S; (void)suh0;
     if (kmask != (1 << 4)) return -4;                          // mixed trellis widths: not built
-    return experts(GLM, x, ldx, R, idx, w, tab, add, out, ws, st);
+    return experts(GLM, x, ldx, R, idx, w, tab, add, out, ws, 0, st);
 }

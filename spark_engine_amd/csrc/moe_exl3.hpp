@@ -1,0 +1,36 @@
+// Shared declarations of the EXL3 MoE translation units.
+#pragma once
+#include "common.hpp"
+
+namespace spk {
+
+enum XType { X_F32 = 0, X_F16 = 1, X_BF16 = 2 };
+
+struct Exl3Cfg {                      // runtime shape of one layer
+    int E, topk, H, I, cbk, act;      // act 0: silu(g) * u, 1: clamp (g <= 10, |u| <= 10) first
+    int xtype, wtype, itype;          // x: XType; route weights: 0 f32, 1 f16; indices: 0 int32, 1 int64
+};
+
+__device__ __forceinline__ float exl3_ld_x(const void* x, int xtype, int64_t i)
+{
+    if (xtype == X_F32) return ((const float*)x)[i];
+    if (xtype == X_F16) return f16_bits_to_f32(((const uint16_t*)x)[i]);
+    return bf16_to_f32(((const uint16_t*)x)[i]);
+}
+__device__ __forceinline__ int exl3_ld_idx(const void* idx, int itype, int i) { return itype ? (int)((const int64_t*)idx)[i] : ((const int*)idx)[i]; }
+__device__ __forceinline__ float exl3_ld_w(const void* w, int wtype, int i) { return wtype ? f16_bits_to_f32(((const uint16_t*)w)[i]) : ((const float*)w)[i]; }
+__device__ __forceinline__ float exl3_act(int act, float a, float u)
+{
+    if (act == 1) { a = fminf(a, 10.0f); u = fminf(fmaxf(u, -10.0f), 10.0f); }
+    return a / (1.0f + __expf(-a)) * u;
+}
+
+// the single-launch decode path (moe_exl3_fused.hip): usable for R <= 16 rows and R * topk <= 256 pairs
+bool exl3_fused_ok(const Exl3Cfg& c, int R);
+size_t exl3_fused_ws_bytes(const Exl3Cfg& c, int R);
+// ws counters must be zero on entry (they are zero again when the call has finished); clean = 0 zeroes them first
+int exl3_xcd_probe();
+int exl3_fused_launch(const Exl3Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
+                      int clean, hipStream_t st);
+
+}  // namespace spk

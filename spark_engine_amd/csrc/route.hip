@@ -8,90 +8,72 @@ using namespace spk;
 
 namespace {
 
-constexpr int ROUTE_EMAX = 1024;   // experts per row a wave can hold (16 per lane)
+constexpr int ROUTE_EMAX = 1024;   // experts per row (one thread each)
 constexpr int ROUTE_KMAX = 16;
 
-// wave-wide argmax of (value, id): larger value wins, equal values go to the lower id
-__device__ __forceinline__ void wave_argmax(float& v, int& id)
-{
-#pragma unroll
-    for (int o = 32; o; o >>= 1) {
-        const float ov = __shfl_xor(v, o, 64);
-        const int oi = __shfl_xor(id, o, 64);
-        if (ov > v || (ov == v && oi < id)) { v = ov; id = oi; }
-    }
-}
-
-// One wave per row.  MODE 0: softmax (weights renormalised over the picks); 1: sqrt(softplus) + bias;
-// 2: sigmoid + bias.  sel = value compared, score = value that becomes the weight.
+// One workgroup per row, one thread per expert.  MODE 0: softmax (weights renormalised over the picks);
+// 1: sqrt(softplus) + bias; 2: sigmoid + bias.  sel = value compared, score = value that becomes the weight.
+// Selection by rank: expert e is pick number #{j : sel[j] > sel[e] or (sel[j] == sel[e] and j < e)}, which is the order
+// repeated argmax with ties to the lower id produces, found in one parallel pass over LDS instead of K serial rounds.
 template <int MODE, typename IT>
 __device__ __forceinline__ void route_row(const float* __restrict__ x, const float* __restrict__ bias, IT* __restrict__ idx,
-                                          float* __restrict__ w, int E, int K, float scale, int lane)
+                                          float* __restrict__ w, int E, int K, float scale)
 {
-    constexpr int PER = ROUTE_EMAX / 64;
-    float score[PER], sel[PER];
+    __shared__ __align__(16) float ssel[ROUTE_EMAX];
+    __shared__ float red[16], pick_s[ROUTE_KMAX];
+    __shared__ int pick_i[ROUTE_KMAX];
+    const int e = threadIdx.x, lane = e & 63, wv = e >> 6, nw = blockDim.x >> 6;
+    const bool on = e < E;
+    float score = 0.f, sel = -INFINITY;
     if (MODE == 0) {
-        float m = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < PER; ++i) { const int e = lane + 64 * i; score[i] = e < E ? x[e] : -INFINITY; m = fmaxf(m, score[i]); }
-        m = wave_max(m);
-        float s = 0.f;
-#pragma unroll
-        for (int i = 0; i < PER; ++i) { const int e = lane + 64 * i; score[i] = e < E ? expf(score[i] - m) : 0.f; s += score[i]; }
-        s = wave_sum(s);
-#pragma unroll
-        for (int i = 0; i < PER; ++i) { const int e = lane + 64 * i; score[i] = score[i] / s; sel[i] = e < E ? score[i] : -INFINITY; }
-    } else {
-#pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int e = lane + 64 * i;
-            if (e < E) {
-                const float v = x[e];
-                score[i] = MODE == 1 ? sqrtf(v > 20.f ? v : log1pf(expf(v))) : 1.f / (1.f + expf(-v));
-                sel[i] = score[i] + bias[e];
-                if (sel[i] != sel[i]) sel[i] = -INFINITY;      // a NaN never wins
-            } else { score[i] = 0.f; sel[i] = -INFINITY; }
-        }
+        const float xv = on ? x[e] : -INFINITY;
+        float m = wave_max(xv);
+        if (lane == 0) red[wv] = m;
+        __syncthreads();
+        m = red[0];
+        for (int i = 1; i < nw; ++i) m = fmaxf(m, red[i]);
+        __syncthreads();
+        const float p = on ? expf(xv - m) : 0.f;
+        float s = wave_sum(p);
+        if (lane == 0) red[wv] = s;
+        __syncthreads();
+        s = 0.f;
+        for (int i = 0; i < nw; ++i) s += red[i];
+        score = p / s;
+        sel = on ? score : -INFINITY;
+    } else if (on) {
+        const float v = x[e];
+        score = MODE == 1 ? sqrtf(v > 20.f ? v : log1pf(expf(v))) : 1.f / (1.f + expf(-v));
+        sel = score + bias[e];
+        if (sel != sel) sel = -INFINITY;               // a NaN never wins
     }
-    float picked[ROUTE_KMAX];
-    int pid[ROUTE_KMAX];
-#pragma unroll
-    for (int k = 0; k < ROUTE_KMAX; ++k) {
-        if (k >= K) break;
-        float bv = -INFINITY, bs = 0.f;
-        int bi = 0x7fffffff;
-#pragma unroll
-        for (int i = 0; i < PER; ++i) { const int e = lane + 64 * i; if (e < E && (sel[i] > bv || (sel[i] == bv && e < bi))) { bv = sel[i]; bi = e; bs = score[i]; } }
-        wave_argmax(bv, bi);
-        float s = 0.f;
-#pragma unroll
-        for (int i = 0; i < PER; ++i) if (lane + 64 * i == bi) { s = score[i]; sel[i] = -INFINITY; }
-        (void)bs;
-        picked[k] = __shfl(s, bi & 63, 64);
-        pid[k] = bi;
+    ssel[e] = sel;
+    __syncthreads();
+    int rank = 0;
+    const int E4 = (E + 3) & ~3;                        // blockDim.x >= E4: the tail entries hold -inf
+    for (int j = 0; j < E4; j += 4) {
+        const float4 o = *(const float4*)&ssel[j];
+        rank += (o.x > sel || (o.x == sel && j < e)) + (o.y > sel || (o.y == sel && j + 1 < e)) + (o.z > sel || (o.z == sel && j + 2 < e)) +
+                (o.w > sel || (o.w == sel && j + 3 < e));
     }
-    if (lane == 0) {
+    if (on && rank < K) { pick_i[rank] = e; pick_s[rank] = score; }
+    __syncthreads();
+    if (e < K) {
         float sum = 0.f;
-#pragma unroll
-        for (int k = 0; k < ROUTE_KMAX; ++k) if (k < K) sum += picked[k];
-#pragma unroll
-        for (int k = 0; k < ROUTE_KMAX; ++k) {
-            if (k >= K) break;
-            idx[k] = (IT)pid[k];
-            if (MODE == 0) w[k] = picked[k] / sum;
-            else if (MODE == 1) w[k] = (K > 1 ? picked[k] / (sum + 1e-20f) : picked[k]) * scale;
-            else w[k] = (picked[k] / fmaxf(sum, 1e-20f)) * scale;
-        }
+        for (int k = 0; k < K; ++k) sum += pick_s[k];
+        idx[e] = (IT)pick_i[e];
+        if (MODE == 0) w[e] = pick_s[e] / sum;
+        else if (MODE == 1) w[e] = (K > 1 ? pick_s[e] / (sum + 1e-20f) : pick_s[e]) * scale;
+        else w[e] = (pick_s[e] / fmaxf(sum, 1e-20f)) * scale;
     }
 }
 
 template <int MODE, typename IT>
-__global__ __launch_bounds__(256) void route_kernel(const float* __restrict__ logits, int64_t ld, const float* __restrict__ bias, IT* __restrict__ idx,
-                                                    float* __restrict__ w, int T, int E, int K, float scale)
+__global__ __launch_bounds__(ROUTE_EMAX) void route_kernel(const float* __restrict__ logits, int64_t ld, const float* __restrict__ bias, IT* __restrict__ idx,
+                                                           float* __restrict__ w, int T, int E, int K, float scale)
 {
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (row >= T) return;
-    route_row<MODE, IT>(logits + (int64_t)row * ld, bias, idx + (int64_t)row * K, w + (int64_t)row * K, E, K, scale, lane);
+    const int row = blockIdx.x;
+    route_row<MODE, IT>(logits + (int64_t)row * ld, bias, idx + (int64_t)row * K, w + (int64_t)row * K, E, K, scale);
 }
 
 // GLM router logits: partial[(r*E + e)*2 + half] = sum over half of K of h[r, k] * W[e, k], binary32 fma.
@@ -127,15 +109,17 @@ __global__ __launch_bounds__(256) void glm_logits_kernel(const float* __restrict
         }
     }
 }
-__global__ __launch_bounds__(64) void glm_select_kernel(const float* __restrict__ partial, const float* __restrict__ bias, long long* __restrict__ ids,
-                                                        float* __restrict__ weights, int experts, int K, float scaling)
+__global__ __launch_bounds__(ROUTE_EMAX) void glm_select_kernel(const float* __restrict__ partial, const float* __restrict__ bias, long long* __restrict__ ids,
+                                                                float* __restrict__ weights, int experts, int K, float scaling)
 {
     __shared__ float lg[ROUTE_EMAX];
-    const int r = blockIdx.x, lane = threadIdx.x;
-    for (int e = lane; e < experts; e += 64) lg[e] = partial[((int64_t)r * experts + e) * 2] + partial[((int64_t)r * experts + e) * 2 + 1];
+    const int r = blockIdx.x, e = threadIdx.x;
+    if (e < experts) lg[e] = partial[((int64_t)r * experts + e) * 2] + partial[((int64_t)r * experts + e) * 2 + 1];
     __syncthreads();
-    route_row<2, long long>(lg, bias, ids + (int64_t)r * K, weights + (int64_t)r * K, experts, K, scaling, lane);
+    route_row<2, long long>(lg, bias, ids + (int64_t)r * K, weights + (int64_t)r * K, experts, K, scaling);
 }
+
+inline int route_threads(int E) { return (E + 63) & ~63; }
 
 }  // namespace
 
@@ -146,7 +130,7 @@ SPARK_API int spark_softmax_route(const void* logits, int64_t ld, int R, int E, 
 {
     if (R < 1) return 0;
     if (E < 1 || E > ROUTE_EMAX || topk < 1 || topk > ROUTE_KMAX || topk > E || ld < E) return 1;
-    route_kernel<0, int><<<(R + 3) / 4, 256, 0, st>>>((const float*)logits, ld, nullptr, (int*)idx, (float*)w, R, E, topk, 1.0f);
+    route_kernel<0, int><<<R, route_threads(E), 0, st>>>((const float*)logits, ld, nullptr, (int*)idx, (float*)w, R, E, topk, 1.0f);
     return launch_status();
 }
 // reference qwen_moe.cu:88-100: 512 experts, top-10
@@ -163,7 +147,7 @@ SPARK_API int ds41_route(const float* logits, const float* bias, int64_t* idx, f
 {
     if (T < 1) return 0;
     if (E < 1 || E > ROUTE_EMAX || K > ROUTE_KMAX || K < 1 || K > E) return 1;
-    route_kernel<1, long long><<<(T + 3) / 4, 256, 0, st>>>(logits, E, bias, (long long*)idx, w, T, E, K, scale);
+    route_kernel<1, long long><<<T, route_threads(E), 0, st>>>(logits, E, bias, (long long*)idx, w, T, E, K, scale);
     return launch_status();
 }
 // sigmoid + bias selection on ready logits f32 [T, E]
@@ -171,7 +155,7 @@ SPARK_API int spark_sigmoid_route(const float* logits, const float* bias, int64_
 {
     if (T < 1) return 0;
     if (E < 1 || E > ROUTE_EMAX || K > ROUTE_KMAX || K < 1 || K > E) return 1;
-    route_kernel<2, long long><<<(T + 3) / 4, 256, 0, st>>>(logits, E, bias, (long long*)idx, w, T, E, K, scaling);
+    route_kernel<2, long long><<<T, route_threads(E), 0, st>>>(logits, E, bias, (long long*)idx, w, T, E, K, scaling);
     return launch_status();
 }
 // reference dataflow.cu:519-546: h f32 [rows, k], w f32 or bf16 [experts, k], partial f32 [rows, experts, 2] scratch
@@ -183,6 +167,6 @@ SPARK_API int glm53_router_fused_cuda(const float* h, const void* w, int w_bf16,
     const unsigned g = (unsigned)((experts * 2 + 3) / 4);
     if (w_bf16) glm_logits_kernel<uint16_t><<<g, 256, 0, st>>>(h, (const uint16_t*)w, partial, rows, experts, k);
     else glm_logits_kernel<float><<<g, 256, 0, st>>>(h, (const float*)w, partial, rows, experts, k);
-    glm_select_kernel<<<rows, 64, 0, st>>>(partial, bias, ids, weights, experts, 8, scaling);
+    glm_select_kernel<<<rows, route_threads(experts), 0, st>>>(partial, bias, ids, weights, experts, 8, scaling);
     return launch_status();
 }

@@ -307,15 +307,24 @@ def exl3_moe_ws(R, H, I, E, topk):
     return n
 
 
-def exl3_moe(x, idx, w, table, H, I, codebook=2, act=0, add=None, out=None, ws=None):
+def exl3_moe_ws_alloc(R, H, I, E, topk, device="cuda:0"):
+    """A workspace zeroed once (spark_exl3_moe_ws_init): calls that pass it with ws_clean=True skip their zeroing launch."""
+    ws = torch.empty(exl3_moe_ws(R, H, I, E, topk), dtype=torch.uint8, device=device)
+    _ck(_lib().spark_exl3_moe_ws_init(_p(ws), ws.numel(), _st()), "spark_exl3_moe_ws_init")
+    return ws
+
+
+def exl3_moe(x, idx, w, table, H, I, codebook=2, act=0, add=None, out=None, ws=None, ws_clean=False, multi_kernel=False):
     """x [R, H] f32 | f16 | bf16, idx int32 | int64 [R, topk], w f32 | f16 [R, topk] -> out f32 [R, H]."""
     R, topk = idx.shape
     if out is None:
         out = torch.empty(R, H, dtype=torch.float32, device=x.device)
     if ws is None:
         ws = torch.empty(exl3_moe_ws(R, H, I, table.E, topk), dtype=torch.uint8, device=x.device)
+        ws_clean = False
+    flags = (1 if ws_clean else 0) | (2 if multi_kernel else 0)
     _ck(_lib().spark_exl3_moe(_p(x), _XT[x.dtype], x.stride(0), R, _p(_dev(idx)), int(idx.dtype == torch.int64), _p(_dev(w)), int(w.dtype == torch.float16),
-                              _p(table.tab), _p(add), _p(out), _p(ws), H, I, table.E, topk, codebook, act, _st()), "spark_exl3_moe")
+                              _p(table.tab), _p(add), _p(out), _p(ws), H, I, table.E, topk, codebook, act, flags, _st()), "spark_exl3_moe")
     return out
 
 

@@ -96,6 +96,26 @@ def test_reference_symbols_qwen_and_glm(ops, oracle):
     assert rel_l2(out, ref) <= TOL
 
 
+@pytest.mark.parametrize("R", [1, 4])
+def test_single_launch_and_multi_kernel_paths_agree(ops, oracle, R):
+    # the decode path runs as one launch; the multi-kernel path (used beyond 16 rows) must give the same values within
+    # FP32 summation order, and a zeroed workspace can be reused call after call (counters clear themselves)
+    g = synth.rng(420 + R)
+    H, I, E, topk = 2048, 512, 64, 10
+    experts = _layer(g, range(E), H, I)
+    table = ops.ExpertTable(_to_dev(experts), E)
+    ws = ops.exl3_moe_ws_alloc(R, H, I, E, topk)
+    for it in range(3):
+        logits = g.standard_normal((R, E)).astype(np.float32)
+        idx, w = oracle.qwen_route(logits, topk)
+        xb = synth.randn_bf16(g, (R, H))
+        ref = oracle.exl3_moe(synth.bf16_to_f32(xb), idx, w, experts, E, H, I, 4, 2, 0)
+        a = host(ops.exl3_moe(dev_bf16(xb), dev(idx), dev(w), table, H, I, ws=ws, ws_clean=True))
+        b = host(ops.exl3_moe(dev_bf16(xb), dev(idx), dev(w), table, H, I, multi_kernel=True))
+        assert rel_l2(a, ref) <= TOL and rel_l2(b, ref) <= TOL
+        assert rel_l2(a, b) <= 3e-4                                      # fp16 roundings of the transformed activations can flip with the summation order
+
+
 def test_exl3_moe_rejects_bad_shapes(ops):
     x = torch.zeros(1, 200, device=DEV)
     with pytest.raises(ops.KernelError):
