@@ -8,72 +8,113 @@ using namespace spk;
 
 namespace {
 
-constexpr int ROUTE_EMAX = 1024;   // experts per row (one thread each)
+constexpr int ROUTE_EMAX = 1024;   // experts per row (16 per lane of one wave)
 constexpr int ROUTE_KMAX = 16;
 
-// One workgroup per row, one thread per expert.  MODE 0: softmax (weights renormalised over the picks);
-// 1: sqrt(softplus) + bias; 2: sigmoid + bias.  sel = value compared, score = value that becomes the weight.
-// Selection by rank: expert e is pick number #{j : sel[j] > sel[e] or (sel[j] == sel[e] and j < e)}, which is the order
-// repeated argmax with ties to the lower id produces, found in one parallel pass over LDS instead of K serial rounds.
-template <int MODE, typename IT>
-__device__ __forceinline__ void route_row(const float* __restrict__ x, const float* __restrict__ bias, IT* __restrict__ idx,
-                                          float* __restrict__ w, int E, int K, float scale)
+// ---- wave64 all-reduce with DPP (no LDS traffic): butterflies inside each row of 16 lanes, then the four row results are
+// read back as scalars.  The result is wave-uniform.
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false); }
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) { return __uint_as_float(dpp_u32<CTRL>(__float_as_uint(v))); }
+constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E, DPP_ROR4 = 0x124, DPP_ROR8 = 0x128;   // quad_perm [1,0,3,2], [2,3,0,1]; row_ror:4, row_ror:8
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v)
 {
-    __shared__ __align__(16) float ssel[ROUTE_EMAX];
-    __shared__ float red[16], pick_s[ROUTE_KMAX];
-    __shared__ int pick_i[ROUTE_KMAX];
-    const int e = threadIdx.x, lane = e & 63, wv = e >> 6, nw = blockDim.x >> 6;
-    const bool on = e < E;
-    float score = 0.f, sel = -INFINITY;
+    v = max(v, dpp_u32<DPP_XOR1>(v)); v = max(v, dpp_u32<DPP_XOR2>(v));
+    v = max(v, dpp_u32<DPP_ROR4>(v)); v = max(v, dpp_u32<DPP_ROR8>(v));
+    const uint32_t a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16), c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    return max(max(a, b), max(c, d));
+}
+__device__ __forceinline__ float readlane_f(float v, int l) { return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), l)); }
+// fixed summation tree: the result is the same on every lane and from call to call
+__device__ __forceinline__ float wave_fsum(float v)
+{
+    v += dpp_f32<DPP_XOR1>(v); v += dpp_f32<DPP_XOR2>(v);
+    v += dpp_f32<DPP_ROR4>(v); v += dpp_f32<DPP_ROR8>(v);
+    const float a = readlane_f(v, 0), b = readlane_f(v, 16), c = readlane_f(v, 32), d = readlane_f(v, 48);
+    return (a + b) + (c + d);
+}
+// order-preserving map of a float to an unsigned integer (-0 treated as +0)
+__device__ __forceinline__ uint32_t fkey(float f)
+{
+    const uint32_t u = __float_as_uint(f + 0.0f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// One wave per row; lane l holds experts l * PER .. l * PER + PER - 1 in registers.  MODE 0: softmax (weights renormalised
+// over the picks); 1: sqrt(softplus) + bias; 2: sigmoid + bias.  sel = value compared, score = value that becomes the
+// weight.  K rounds of argmax: the largest key by a DPP reduction, then the lowest lane holding it (a ballot) and that
+// lane's lowest expert with it: ties go to the lower expert id.
+template <int MODE, int PER, typename IT>
+__device__ __forceinline__ void route_row(const float* __restrict__ x, const float* __restrict__ bias, IT* __restrict__ idx,
+                                          float* __restrict__ w, int E, int K, float scale, int lane)
+{
+    float score[PER];
+    uint32_t key[PER];                                   // 0 = not a candidate (absent, taken, or NaN)
+    const int e0 = lane * PER;
     if (MODE == 0) {
-        const float xv = on ? x[e] : -INFINITY;
-        float m = wave_max(xv);
-        if (lane == 0) red[wv] = m;
-        __syncthreads();
-        m = red[0];
-        for (int i = 1; i < nw; ++i) m = fmaxf(m, red[i]);
-        __syncthreads();
-        const float p = on ? expf(xv - m) : 0.f;
-        float s = wave_sum(p);
-        if (lane == 0) red[wv] = s;
-        __syncthreads();
-        s = 0.f;
-        for (int i = 0; i < nw; ++i) s += red[i];
-        score = p / s;
-        sel = on ? score : -INFINITY;
-    } else if (on) {
-        const float v = x[e];
-        score = MODE == 1 ? sqrtf(v > 20.f ? v : log1pf(expf(v))) : 1.f / (1.f + expf(-v));
-        sel = score + bias[e];
-        if (sel != sel) sel = -INFINITY;               // a NaN never wins
+        float xv[PER], m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) { xv[i] = e0 + i < E ? x[e0 + i] : -INFINITY; m = fmaxf(m, xv[i]); }
+        // wave maximum through the ordered keys
+        {
+            const uint32_t km = wave_umax(fkey(m));
+            m = __uint_as_float((km & 0x80000000u) ? (km & 0x7fffffffu) : ~km);
+        }
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) { score[i] = e0 + i < E ? expf(xv[i] - m) : 0.f; s += score[i]; }
+        s = wave_fsum(s);
+#pragma unroll
+        for (int i = 0; i < PER; ++i) { score[i] = score[i] / s; key[i] = e0 + i < E ? fkey(score[i]) : 0u; }
+    } else {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            score[i] = 0.f; key[i] = 0u;
+            if (e0 + i < E) {
+                const float v = x[e0 + i];
+                score[i] = MODE == 1 ? sqrtf(v > 20.f ? v : log1pf(expf(v))) : 1.f / (1.f + expf(-v));
+                const float sel = score[i] + bias[e0 + i];
+                key[i] = sel != sel ? 1u : max(fkey(sel), 1u);      // a NaN never wins over a number; -inf still ranks above "absent"
+            }
+        }
     }
-    ssel[e] = sel;
-    __syncthreads();
-    int rank = 0;
-    const int E4 = (E + 3) & ~3;                        // blockDim.x >= E4: the tail entries hold -inf
-    for (int j = 0; j < E4; j += 4) {
-        const float4 o = *(const float4*)&ssel[j];
-        rank += (o.x > sel || (o.x == sel && j < e)) + (o.y > sel || (o.y == sel && j + 1 < e)) + (o.z > sel || (o.z == sel && j + 2 < e)) +
-                (o.w > sel || (o.w == sel && j + 3 < e));
+    float mine = 0.f, sum = 0.f;                          // lane k keeps pick k
+    int mine_id = 0;
+    for (int k = 0; k < K; ++k) {
+        uint32_t bk = 0u; int bi = 0;
+#pragma unroll
+        for (int i = PER - 1; i >= 0; --i) if (key[i] >= bk) { bk = key[i]; bi = i; }   // lowest i among equals
+        const uint32_t wk = wave_umax(bk);
+        const uint64_t bal = __builtin_amdgcn_ballot_w64(bk == wk);
+        const int wl = __builtin_ctzll(bal);               // lowest lane = lowest expert ids
+        const int wi = __builtin_amdgcn_readlane(bi, wl);
+        float sc = 0.f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) if (lane == wl && i == wi) { sc = score[i]; key[i] = 0u; }
+        sc = readlane_f(sc, wl);
+        sum += sc;
+        if (lane == k) { mine = sc; mine_id = wl * PER + wi; }
     }
-    if (on && rank < K) { pick_i[rank] = e; pick_s[rank] = score; }
-    __syncthreads();
-    if (e < K) {
-        float sum = 0.f;
-        for (int k = 0; k < K; ++k) sum += pick_s[k];
-        idx[e] = (IT)pick_i[e];
-        if (MODE == 0) w[e] = pick_s[e] / sum;
-        else if (MODE == 1) w[e] = (K > 1 ? pick_s[e] / (sum + 1e-20f) : pick_s[e]) * scale;
-        else w[e] = (pick_s[e] / fmaxf(sum, 1e-20f)) * scale;
+    if (lane < K) {
+        idx[lane] = (IT)mine_id;
+        if (MODE == 0) w[lane] = mine / sum;
+        else if (MODE == 1) w[lane] = (K > 1 ? mine / (sum + 1e-20f) : mine) * scale;
+        else w[lane] = (mine / fmaxf(sum, 1e-20f)) * scale;
     }
 }
 
-template <int MODE, typename IT>
-__global__ __launch_bounds__(ROUTE_EMAX) void route_kernel(const float* __restrict__ logits, int64_t ld, const float* __restrict__ bias, IT* __restrict__ idx,
-                                                           float* __restrict__ w, int T, int E, int K, float scale)
+template <int MODE, int PER, typename IT>
+__global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ logits, int64_t ld, const float* __restrict__ bias, IT* __restrict__ idx,
+                                                   float* __restrict__ w, int T, int E, int K, float scale)
 {
     const int row = blockIdx.x;
-    route_row<MODE, IT>(logits + (int64_t)row * ld, bias, idx + (int64_t)row * K, w + (int64_t)row * K, E, K, scale);
+    route_row<MODE, PER, IT>(logits + (int64_t)row * ld, bias, idx + (int64_t)row * K, w + (int64_t)row * K, E, K, scale, threadIdx.x);
+}
+template <int MODE, typename IT>
+void launch_route(const float* logits, int64_t ld, const float* bias, IT* idx, float* w, int T, int E, int K, float scale, hipStream_t st)
+{
+    if (E <= 256) route_kernel<MODE, 4, IT><<<T, 64, 0, st>>>(logits, ld, bias, idx, w, T, E, K, scale);
+    else if (E <= 512) route_kernel<MODE, 8, IT><<<T, 64, 0, st>>>(logits, ld, bias, idx, w, T, E, K, scale);
+    else route_kernel<MODE, 16, IT><<<T, 64, 0, st>>>(logits, ld, bias, idx, w, T, E, K, scale);
 }
 
 // GLM router logits: partial[(r*E + e)*2 + half] = sum over half of K of h[r, k] * W[e, k], binary32 fma.
@@ -109,17 +150,15 @@ __global__ __launch_bounds__(256) void glm_logits_kernel(const float* __restrict
         }
     }
 }
-__global__ __launch_bounds__(ROUTE_EMAX) void glm_select_kernel(const float* __restrict__ partial, const float* __restrict__ bias, long long* __restrict__ ids,
-                                                                float* __restrict__ weights, int experts, int K, float scaling)
+__global__ __launch_bounds__(64) void glm_select_kernel(const float* __restrict__ partial, const float* __restrict__ bias, long long* __restrict__ ids,
+                                                        float* __restrict__ weights, int experts, int K, float scaling)
 {
-    __shared__ float lg[ROUTE_EMAX];
-    const int r = blockIdx.x, e = threadIdx.x;
-    if (e < experts) lg[e] = partial[((int64_t)r * experts + e) * 2] + partial[((int64_t)r * experts + e) * 2 + 1];
+    __shared__ float lg[320];
+    const int r = blockIdx.x, lane = threadIdx.x;
+    for (int e = lane; e < experts; e += 64) lg[e] = partial[((int64_t)r * experts + e) * 2] + partial[((int64_t)r * experts + e) * 2 + 1];
     __syncthreads();
-    route_row<2, long long>(lg, bias, ids + (int64_t)r * K, weights + (int64_t)r * K, experts, K, scaling);
+    route_row<2, 5, long long>(lg, bias, ids + (int64_t)r * K, weights + (int64_t)r * K, experts, K, scaling, lane);
 }
-
-inline int route_threads(int E) { return (E + 63) & ~63; }
 
 }  // namespace
 
@@ -130,7 +169,7 @@ SPARK_API int spark_softmax_route(const void* logits, int64_t ld, int R, int E, 
 {
     if (R < 1) return 0;
     if (E < 1 || E > ROUTE_EMAX || topk < 1 || topk > ROUTE_KMAX || topk > E || ld < E) return 1;
-    route_kernel<0, int><<<R, route_threads(E), 0, st>>>((const float*)logits, ld, nullptr, (int*)idx, (float*)w, R, E, topk, 1.0f);
+    launch_route<0, int>((const float*)logits, ld, nullptr, (int*)idx, (float*)w, R, E, topk, 1.0f, st);
     return launch_status();
 }
 // reference qwen_moe.cu:88-100: 512 experts, top-10
@@ -147,7 +186,7 @@ SPARK_API int ds41_route(const float* logits, const float* bias, int64_t* idx, f
 {
     if (T < 1) return 0;
     if (E < 1 || E > ROUTE_EMAX || K > ROUTE_KMAX || K < 1 || K > E) return 1;
-    route_kernel<1, long long><<<T, route_threads(E), 0, st>>>(logits, E, bias, (long long*)idx, w, T, E, K, scale);
+    launch_route<1, long long>(logits, E, bias, (long long*)idx, w, T, E, K, scale, st);
     return launch_status();
 }
 // sigmoid + bias selection on ready logits f32 [T, E]
@@ -155,7 +194,7 @@ SPARK_API int spark_sigmoid_route(const float* logits, const float* bias, int64_
 {
     if (T < 1) return 0;
     if (E < 1 || E > ROUTE_EMAX || K > ROUTE_KMAX || K < 1 || K > E) return 1;
-    route_kernel<2, long long><<<T, route_threads(E), 0, st>>>(logits, E, bias, (long long*)idx, w, T, E, K, scaling);
+    launch_route<2, long long>(logits, E, bias, (long long*)idx, w, T, E, K, scaling, st);
     return launch_status();
 }
 // reference dataflow.cu:519-546: h f32 [rows, k], w f32 or bf16 [experts, k], partial f32 [rows, experts, 2] scratch
@@ -167,6 +206,6 @@ SPARK_API int glm53_router_fused_cuda(const float* h, const void* w, int w_bf16,
     const unsigned g = (unsigned)((experts * 2 + 3) / 4);
     if (w_bf16) glm_logits_kernel<uint16_t><<<g, 256, 0, st>>>(h, (const uint16_t*)w, partial, rows, experts, k);
     else glm_logits_kernel<float><<<g, 256, 0, st>>>(h, (const float*)w, partial, rows, experts, k);
-    glm_select_kernel<<<rows, route_threads(experts), 0, st>>>(partial, bias, ids, weights, experts, 8, scaling);
+    glm_select_kernel<<<rows, 64, 0, st>>>(partial, bias, ids, weights, experts, 8, scaling);
     return launch_status();
 }
