@@ -1,0 +1,174 @@
+/* C ABI of libspark_shim_hip.so: the MI355X (gfx950) build of spark-engine's quantized MoE expert path.
+ *
+ * Every entry point keeps the reference shim's contract (engine-rs/shim): plain device pointers, a trailing stream, `int` return
+ * with 0 = success (a small positive / negative code for argument errors, otherwise the hipError_t of the launch), no allocation and
+ * no synchronisation inside, every scratch buffer passed in by the caller and sized by the matching *_ws_bytes, fixed grids with
+ * device-side counts so a call can be recorded into a HIP graph.  Results are deterministic and independent of the number of rows in
+ * the call.  `hipStream_t` replaces `cudaStream_t` in the position the reference has it.
+ *
+ * Names that start with `qwen_`, `glm`, `ds41_` are the reference's own symbols (same parameter order and meaning); each comment
+ * names the reference definition it replaces.  Names that start with `spark_` are run-time-sized forms of the same kernels that the
+ * reference does not export (its dimensions are compile-time traits).
+ */
+#ifndef SPARK_SHIM_H
+#define SPARK_SHIM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#ifndef SPARK_API
+#define SPARK_API
+#endif
+#ifndef HIP_INCLUDE_HIP_HIP_RUNTIME_API_H
+typedef struct ihipStream_t* hipStream_t;
+#endif
+
+/* ---------------------------------------------------------------- dequantisation surfaces (bit-exact) ------------------------ */
+
+/* EXL3 trellis [K/16, N/16, 16*bits] int16 -> the inner matrix [K, N] fp16 (no Hadamard, no scales); bits 3..6;
+ * codebook 1 = mcg, 2 = mul1.  Replaces engine-rs/shim/qwen_exl3.cu:221 (qwen_exl3_reconstruct, mul1 only). */
+SPARK_API int spark_exl3_reconstruct(const void* trellis, void* w_f16, int K, int N, int bits, int codebook, hipStream_t st);
+SPARK_API int qwen_exl3_reconstruct(const void* trellis, void* w_f16, int K, int N, int bits, hipStream_t st);
+/* Effective weight W = diag(suh) H inner H diag(svh), written transposed [N, K] fp16 with row stride ldo.
+ * Replaces engine-rs/shim/qwen_exl3.cu:208 (qwen_exl3_fold). */
+SPARK_API int spark_exl3_fold(const void* trellis, const void* suh, const void* svh, int K, int N, int bits, int codebook, void* out_f16,
+                              int64_t ldo, hipStream_t st);
+SPARK_API int qwen_exl3_fold(const void* trellis, const void* suh, const void* svh, int K, int N, int bits, void* out_f16, int64_t ldo,
+                             hipStream_t st);
+/* MXFP4: w [N, K/2] bytes (low nibble = even k), s [N, K/32] E8M0 -> fp32 [N, K].
+ * Restates reference/ds41/kernel.py:122-131 (dequant_fp4_weight) and engine-rs/src/ds41/load.rs:338-349. */
+SPARK_API int spark_mxfp4_dequant(const void* w, const void* s, float* out, int N, int K, hipStream_t st);
+/* FP8 E4M3 [N, K] with one fp32 scale per bs x bs block -> fp32.  Restates reference/ds41/kernel.py:96-99. */
+SPARK_API int spark_fp8_block_dequant(const void* w, const float* s, float* out, int N, int K, int bs, hipStream_t st);
+/* FP8 E4M3 [N, K] with one E8M0 scale per 32 x 32 block (the engine's dense layout, engine-rs/shim/ds41.cu:28-73) -> fp32. */
+SPARK_API int spark_fp8_e8m0_dequant(const void* w, const void* s, float* out, int N, int K, hipStream_t st);
+
+/* ---------------------------------------------------------------- activation quantisation and glue -------------------------- */
+
+/* x bf16 -> per 32: power-of-two scale from the block maximum, E4M3 round-to-nearest-even saturating, dequantised back to bf16.
+ * Replaces engine-rs/shim/ds41.cu:274 (ds41_act_quant32); bit-exact with engine-rs/src/ds41/ops.rs:26-35. */
+SPARK_API int ds41_act_quant32(const void* x, void* out, long long numel, hipStream_t st);
+/* Same quantiser, leaving the E4M3 bytes q [numel] and the E8M0 scale bytes s [numel/32].  Replaces ds41_mx.cu:1406. */
+SPARK_API int ds41_act_quant_fp8(const void* x, void* q, void* s, long long numel, hipStream_t st);
+/* gu fp32 [T, 2I] (gate | up) -> act_quant(bf16(silu(min(g, lim)) * clamp(u, +-lim))) bf16 [T, I].  Replaces ds41_ops.cu:615. */
+SPARK_API int ds41_swiglu_quant(const float* gu, void* out, int T, int I, float lim, hipStream_t st);
+/* h = silu(g) * u over n fp32 values.  Replaces engine-rs/shim/qwen_moe.cu:101. */
+SPARK_API int qwen_moe_silu_mul(const void* g, const void* u, void* h, int n, hipStream_t st);
+/* out[r, :] = sigmoid(gl[r * ldg + col]) * d[r, :] (the shared expert's scalar gate).  Replaces qwen_moe.cu:106. */
+SPARK_API int qwen_moe_gate_scale(const void* gl, int64_t ldg, int col, const void* d, void* out, int R, int N, hipStream_t st);
+
+/* ---------------------------------------------------------------- routers ---------------------------------------------------- */
+
+/* softmax over E fp32 logits (row stride ld), top-k by repeated argmax with ties to the lower index, weights renormalised to sum 1.
+ * idx int32 [R, topk], w fp32 [R, topk].  E <= 1024, topk <= 16.  Replaces engine-rs/shim/qwen_moe.cu:10-66,90-99. */
+SPARK_API int spark_softmax_route(const void* logits, int64_t ld, int R, int E, int topk, void* idx, void* w, hipStream_t st);
+SPARK_API int qwen_moe_route(const void* logits, int R, void* idx, void* w, hipStream_t st);
+SPARK_API int qwen_moe_route_ld(const void* logits, int64_t ld, int R, void* idx, void* w, hipStream_t st);
+/* s = sqrt(softplus(x)), top-K of s + bias, w = s / (sum + 1e-20) * scale for K > 1.  idx int64 [T, K].
+ * Replaces engine-rs/shim/ds41_ops.cu:376-419,609. */
+SPARK_API int ds41_route(const float* logits, const float* bias, int64_t* idx, float* w, int T, int E, int K, float scale, hipStream_t st);
+/* score = sigmoid(x), top-K of score + bias, w = score / max(sum, 1e-20) * scaling.  Restates dataflow.cu:433-448,489-513. */
+SPARK_API int spark_sigmoid_route(const float* logits, const float* bias, int64_t* idx, float* w, int T, int E, int K, float scaling,
+                                  hipStream_t st);
+/* GLM router: logits = h [rows, k] fp32 x w [experts, k] (fp32 or bf16), then the sigmoid selection above.
+ * `partial` is scratch of rows * experts * glm53_router_split() floats.  Replaces engine-rs/shim/dataflow.cu:519-546. */
+SPARK_API int glm53_router_split(void);
+SPARK_API int glm53_router_fused_cuda(const float* h, const void* w, int w_bf16, const float* bias, float* partial, long long* ids,
+                                      float* weights, int rows, int experts, int k, float scaling, hipStream_t st);
+
+/* ---------------------------------------------------------------- dense quantised GEMVs (m <= 8 rows) ----------------------- */
+
+/* y [m, n] fp32 = x [m, k] bf16 . w^T, w [n, k/2] MXFP4 codes, ws [n, k/32] E8M0.  Replaces engine-rs/shim/ds41.cu:75-110,236. */
+SPARK_API int ds41_mxfp4_gemv(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, hipStream_t st);
+/* w [n, k] E4M3 with E8M0 scales per 32 x 32 block; xs = row stride of x in elements; rpg = rows per scale group of a stacked
+ * weight (0 = one matrix).  Replaces engine-rs/shim/ds41.cu:28-73,240,248. */
+SPARK_API int ds41_fp8_gemv_ex(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, int xs, int rpg, hipStream_t st);
+SPARK_API int ds41_fp8_gemv(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, hipStream_t st);
+/* w [n, k] E4M3 with fp32 scales [ceil(n/128), ceil(k/128)]; the projection of reference/ds41/kernel.py:96-119 (fp8_gemm) with bf16
+ * activations used as given. */
+SPARK_API int spark_fp8_block128_gemv(const void* x, const void* w, const float* scales, float* y, int m, int n, int k, hipStream_t st);
+/* w [n, k] bf16 (router logits).  Replaces engine-rs/shim/ds41.cu:252. */
+SPARK_API int ds41_bf16_gemv(const void* x, const void* w, float* y, int m, int n, int k, hipStream_t st);
+
+/* ---------------------------------------------------------------- MXFP4 expert layer ---------------------------------------- */
+
+/* y[r] = add[r] + sum over shared experts + sum_k (slot order) w2_e . q(bf16(silu(min(bf16(w1_e . xq), 10)) * clamp(bf16(w3_e . xq), +-10)
+ * * rw[r, k])), q = the act_quant above, products against E4M3 activations with E8M0 scales exact in fp32
+ * (engine-rs/shim/ds41_moe.cu:1-24, ds41_mx.cu:129-292).
+ * layout: 0 = streaming records made by spark_mxfp4_prepack, 1 = checkpoint layout w [E, rows, K/2] + s [E, rows, K/32],
+ *         2 = the reference's moe_pack layout (engine-rs/src/ds41/kern.rs:718-726), 3 = its moe_pack_mx layout (kern.rs:728-734).
+ * Shared experts (n_shared of them, weight 1, every row) are experts E .. E + n_shared - 1 of the same stacked tensors. */
+SPARK_API size_t spark_mxfp4_packed_bytes(long long rows_total, int K);
+SPARK_API int spark_mxfp4_prepack(const void* w, const void* s, void* packed, long long rows_total, int K, hipStream_t st);
+SPARK_API size_t spark_mxfp4_moe_ws_bytes(int R, int H, int I, int topk, int E, int n_shared);
+/* xq E4M3 [R, H], xs E8M0 [R, H/32] */
+SPARK_API int spark_mxfp4_moe_q(const void* xq, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1,
+                                const void* w3, const void* s3, const void* w2, const void* s2, int layout, int H, int I, int topk, int E,
+                                int n_shared, const float* add, float* y, void* ws, hipStream_t st);
+/* x bf16 [R, H]; xq / xs are caller scratch of R*H and R*H/32 bytes */
+SPARK_API int spark_mxfp4_moe(const void* x, void* xq, void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1,
+                              const void* w3, const void* s3, const void* w2, const void* s2, int layout, int H, int I, int topk, int E,
+                              int n_shared, const float* add, float* y, void* ws, hipStream_t st);
+/* The reference's DeepSeek entry points (H = 5120 as compiled there, weights in the moe_pack_mx layout with raw scale bytes).
+ * Replace engine-rs/shim/ds41_mx.cu:1426-1523.  ds41_moe_mx_ws_ptrs hands out the per-pair down output [P, H] fp32 and pairmap [P]
+ * inside ws, valid after ds41_moe_mx_ex(skip_combine = 1). */
+SPARK_API void ds41_moe_mx_set_s2(int on);
+SPARK_API int ds41_moe_mx_get_s2(void);
+SPARK_API void ds41_moe_gr16_max(int v);
+SPARK_API int ds41_moe_mx_col_passes(int R, int topk, int E);
+SPARK_API int ds41_moe_mx_pair_b16(int R, int topk, int E);
+SPARK_API size_t ds41_moe_mx_ws_bytes(int R, int I, int topk, int E);
+SPARK_API int ds41_moe_mx_ex(const void* xq, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1,
+                             const void* w3, const void* s3, const void* w2, const void* s2, int I, const float* add, float* y, void* ws,
+                             int topk, int E, int skip_combine, hipStream_t st);
+SPARK_API int ds41_moe_mx(const void* xq, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1,
+                          const void* w3, const void* s3, const void* w2, const void* s2, int I, const float* add, float* y, void* ws, int topk,
+                          int E, hipStream_t st);
+SPARK_API int ds41_moe_mx_combine_rows(void* ws, int R, int I, int topk, int E, const float* add, float* y, int r0, int nr, hipStream_t st);
+SPARK_API int ds41_moe_mx_combine(void* ws, int R, int I, int topk, int E, const float* add, float* y, hipStream_t st);
+SPARK_API int ds41_moe_mx_ws_ptrs(void* ws, int R, int I, int topk, int E, float** out, int** pairmap);
+/* bf16 activations (already act-quantised), weights in the moe_pack layout.  Replaces engine-rs/shim/ds41_moe.cu:259-292. */
+SPARK_API size_t ds41_moe_ws_bytes(int R, int I, int topk, int E);
+SPARK_API int ds41_moe(const void* xq, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3,
+                       const void* s3, const void* w2, const void* s2, int I, const float* add, float* y, void* ws, int topk, int E,
+                       hipStream_t st);
+
+/* ---------------------------------------------------------------- EXL3 expert layer ----------------------------------------- */
+
+/* out[r] = add[r] + sum_k (slot order) w[r, k] * down_e(act(gate_e(x_r), up_e(x_r))), every matrix an EXL3 4-bit trellis with its
+ * own Hadamard sign vector suh [K] and channel scale svh [N] (fp16).  tab = uint64 [9][E] device pointers: gate, up, down trellis;
+ * gate, up, down suh; gate, up, down svh (engine-rs/shim/moe_exl3.cuh:8-9).  xtype / wtype: 0 fp32, 1 fp16, 2 bf16; itype: 0 int32,
+ * 1 int64; act: 0 silu(g) * u, 1 the same after clamping g <= 10 and |u| <= 10; codebook 1 mcg, 2 mul1.  out fp32 [R, H].
+ * flags bit 0: ws was prepared by spark_exl3_moe_ws_init and only ever used by this entry point (skips the clearing launch);
+ * flags bit 1: force the several-kernel path.
+ * Replaces engine-rs/shim/moe_exl3.cuh:1512-1691 (moex::experts). */
+SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk);
+SPARK_API int spark_exl3_moe_ws_init(void* ws, size_t bytes, hipStream_t st);
+SPARK_API int spark_exl3_moe(const void* x, int xtype, int64_t ldx, int R, const void* idx, int itype, const void* w, int wtype, const void* tab,
+                             const void* add, void* out, void* ws, int H, int I, int E, int topk, int codebook, int act, int flags,
+                             hipStream_t st);
+/* Qwen: E 512, top-10, H 2560, I 640, x / w fp32, idx int32, mul1.  Replaces engine-rs/shim/qwen_moe.cu:111-117. */
+SPARK_API size_t qwen_moe_ws_bytes(int R, int S);
+SPARK_API int qwen_moe_experts(const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out,
+                               void* ws, int S, hipStream_t st);
+/* GLM: E 288, top-8, H 4096, I 1024, x / w fp16, idx int64, mcg, clamped activation; kmask must be 1 << 4 (4-bit experts only).
+ * Replaces engine-rs/shim/glm_moe.cu:8-16. */
+SPARK_API size_t glm_moe_ws_bytes(int R, int S);
+SPARK_API int glm_moe_experts(const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out,
+                              void* ws, int S, const void* suh0, int kmask, hipStream_t st);
+
+/* ---------------------------------------------------------------- diagnostics (not part of the reference ABI) ---------------- */
+
+/* buf = device memory of 8 * gridDim int64 the single-launch EXL3 kernel fills with per-block wall-clock stamps (NULL = off) */
+SPARK_API void spark_debug_exl3_trace(long long* buf);
+/* exchange mode of the single-launch EXL3 kernel: 1 = same-XCD through L2, 0 = device-coherent, -1 = measure placement again */
+SPARK_API void spark_debug_exl3_local(int v);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
