@@ -258,7 +258,7 @@ int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, co
     if (!cfg_ok(c, R)) return -1;
     if (!(flags & 2) && exl3_fused_ok(c, R)) return exl3_fused_launch(c, x, ldx, R, idx, w, tab, add, out, ws, flags & 1, st);
     const Plan p = plan(c, R);
-    char* b = (char*)ws;
+    char* b = (char*)ws + (exl3_fused_ok(c, R) ? exl3_fused_ws_bytes(c, R) : 0);       // the two paths never share workspace bytes
     int* G = (int*)(b + p.G);
     int *gexp = (int*)(b + p.gexp), *goff = (int*)(b + p.goff), *gcnt = (int*)(b + p.gcnt);
     int *pairmap = (int*)(b + p.pairmap), *prow = (int*)(b + p.prow), *pexp = (int*)(b + p.pexp);
@@ -298,13 +298,13 @@ SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk)
     const Cfg c{E, topk, H, I, CB_MUL1, 0, 0, 0, 0};
     if (!cfg_ok(c, R)) return 0;
     const size_t a = plan(c, R).total, b = exl3_fused_ok(c, R) ? exl3_fused_ws_bytes(c, R) : 0;
-    return a > b ? a : b;
+    return a + b;
 }
-// zeroes the workspace once after allocation; calls made with flags bit 0 set then skip their own zeroing launch
+// prepares the workspace once after allocation; calls made with flags bit 0 set then skip their own preparing launch
 SPARK_API int spark_exl3_moe_ws_init(void* ws, size_t bytes, hipStream_t st)
 {
     exl3_xcd_probe();                 // one-time placement check (synchronises; this call is made outside stream capture)
-    return (int)hipMemsetAsync(ws, 0, bytes, st);
+    return exl3_fused_ws_prepare(ws, bytes, st);
 }
 SPARK_API int spark_exl3_moe(const void* x, int xtype, int64_t ldx, int R, const void* idx, int itype, const void* w, int wtype, const void* tab,
                              const void* add, void* out, void* ws, int H, int I, int E, int topk, int codebook, int act, int flags, hipStream_t st)

@@ -28,8 +28,10 @@ __device__ __forceinline__ float exl3_act(int act, float a, float u)
 // the single-launch decode path (moe_exl3_fused.hip): usable for R <= 16 rows and R * topk <= 256 pairs
 bool exl3_fused_ok(const Exl3Cfg& c, int R);
 size_t exl3_fused_ws_bytes(const Exl3Cfg& c, int R);
-// ws counters must be zero on entry (they are zero again when the call has finished); clean = 0 zeroes them first
+// The exchanged words of ws must be in their idle state on entry (they are again when the call has finished): clean = 0
+// prepares them first with one more launch.  exl3_fused_ws_prepare does that for a whole buffer, once, after allocation.
 int exl3_xcd_probe();
+int exl3_fused_ws_prepare(void* ws, size_t bytes, hipStream_t st);
 int exl3_fused_launch(const Exl3Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
                       int clean, hipStream_t st);
 

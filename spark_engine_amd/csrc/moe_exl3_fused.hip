@@ -3,25 +3,31 @@
 // The multi-kernel path (moe_exl3.hip) needs seven dependent launches for a layer that moves 16 MB: launch gaps and the
 // chain of cold first loads cost far more than the weight stream.  Here one grid holds both weight streams:
 //   A blocks: (item, 128-column block of I | gate or up, K slice).  Transform the slice of x (x * suh, Hadamard, fp16)
-//       into LDS, stream and decode the slice's k-tiles, write FP32 partials; the last block of an (item, column block)
-//       group sums the slices, finishes gate and up (Hadamard, svh), applies the activation and the down input
-//       transform and publishes that block of xh2; a per-item counter tells the B blocks when all of xh2 is there.
+//       into LDS while the slice's k-tiles stream in, decode, dot, write FP32 partials.  The last block of an
+//       (item, column block) group in launch order is its finisher: it takes the other blocks' partials, finishes gate
+//       and up (Hadamard, svh), applies the activation and the down input transform and hands that block of xh2 to
+//       every down-projection block of the item.
 //   B blocks: (128-column block of H | item, K slice).  Issue and DECODE their down-projection tiles first (they do not
-//       depend on stage 1), then wait for the item's counter, dot with xh2, finish (Hadamard, svh); the block that
-//       completes a token row's last expert does the weighted slot-order sum for its 128 columns.
+//       depend on stage 1), then take the item's xh2, dot, finish (Hadamard, svh).  For every token row the block of
+//       the row's last item in launch order does the weighted slot-order sum for its 128 columns.
+//
+// Exchange without counters: every exchanged 32-bit word of the workspace is EMPTY (all ones) between uses.  A producer
+// simply stores its value (a value that happens to be all ones, one particular NaN, is stored as another NaN); the one
+// consumer of a word polls until it is no longer EMPTY, then stores EMPTY back.  No fence, no acknowledged-store wait and
+// no atomic lies on the critical path: one store and one load per hop.  Every word has exactly one consumer (xh2 is
+// written once per consuming column block for that reason), so the workspace is all EMPTY again when the kernel ends.
 //
 // XCD-aware placement.  MI355X has 8 XCDs with one L2 each, and workgroup b runs on XCD b % 8 (checked once per process
 // by reading XCC_ID).  Block ids are laid out so that every exchange but one stays inside one XCD: the 2 * S1 blocks of
 // an (item, column block) group share an XCD, and so do all B blocks of one output column block (their experts' outputs
-// meet in the final sum).  Inside an XCD data moves through the shared L2 with ordinary stores, L1-bypassing loads and
-// L2 atomics.  Only xh2 crosses XCDs, through device-coherent stores / loads (slow: they go to memory), once per item.
-// If the placement check fails, every exchange uses the device-coherent form.
+// meet in the final sum).  Inside an XCD data moves through the shared L2 with ordinary stores and L1-bypassing loads.
+// Only xh2 crosses XCDs, through device-coherent stores / loads.  If the placement check fails, every exchange uses the
+// device-coherent form.
 //
-// Blocks are dispatched in id order and all A blocks precede all B blocks, so every A block is resident or done before a
-// B block can start waiting; A blocks never wait.  Waits are bounded: on expiry the block sets an error flag and skips
-// its work, and every block still runs to its end, so the grid always drains.  The last block to finish clears the
-// counters for the next call.  A producer block waits until every wave's stores are acknowledged (s_waitcnt vmcnt(0),
-// a workgroup fence does not wait for global stores), then one thread bumps the counter.
+// Progress.  Blocks are dispatched in id order and a block only ever waits for blocks with lower ids (A before B, the
+// finisher is the last block of its group, the summing block belongs to the row's last item), so whatever a block waits
+// for is resident or done.  Waits are bounded: on expiry the block sets an error flag and skips its work, and every
+// block still runs to its end, so the grid always drains (the workspace must then be initialised again).
 //
 // Items are distinct experts in order of first appearance; rows of the per-pair buffers are the pair indices r * topk + k.
 // Semantics: reference engine-rs/shim/moe_exl3.cuh:204-228,272-285,935-956,1019-1064,1084-1112,1380-1410.
@@ -38,74 +44,76 @@ constexpr int FW = 4;                 // waves per block
 constexpr int TW = 8;                 // k-tiles per wave (all loaded up front)
 constexpr int KTB = FW * TW;          // k-tiles per block = K slice of 512
 constexpr int PF_MAX = 256, RF_MAX = 16;
-constexpr int SPIN_MAX = 400000;
+constexpr int SPIN_MAX = 200000;
 constexpr int SMAX = 8;               // K slices per product (K <= 4096)
 constexpr int NXCD = 8;
+constexpr int HEAD = 256;             // bytes at the start of the workspace: [0] error flag (sticky)
+constexpr uint32_t EMPTY = 0xffffffffu;
+constexpr uint64_t EMPTY2 = ~0ull;
 
 struct FArgs {
     const void* x; int64_t ldx; const void* idx; const void* w; const uint64_t* tab; const float* add; float* out;
-    float* part1; uint16_t* xh2; float* part2; float* yd; int* cnt;
-    int R, P, Gmax, S1, S2, NB1, NB2, nA, nB, ncnt, bpgA, bpgB, local;
+    float* part1;                     // [S1][2][P][I] gate / up partial sums per K slice
+    uint32_t* xh2;                    // [NB2][P][I / 2] packed fp16 pairs: one copy of the down input per consuming column block
+    float* part2;                     // [S2][P][H] down partial sums per K slice (S2 > 1 only)
+    float* yd;                        // [P][H] per-pair expert outputs
+    int* err;
+    int R, P, Gmax, S1, S2, NB1, NB2, nA, nB, bpgA, bpgB, local;
     Exl3Cfg c;
     long long* trace;                 // optional per-block timestamps (diagnostics), 8 per block
 };
-// counter layout: [0] XCDs done, [1] error flag (sticky), [2..9] blocks done per XCD, then cnt1 [Gmax][NB1], ready [Gmax],
-// cnt2 [Gmax][NB2], cnt3 [R][NB2]
-__device__ __forceinline__ int* cnt1_of(const FArgs& a) { return a.cnt + 2 + NXCD; }
-__device__ __forceinline__ int* ready_of(const FArgs& a) { return cnt1_of(a) + a.Gmax * a.NB1; }
-__device__ __forceinline__ int* cnt2_of(const FArgs& a) { return ready_of(a) + a.Gmax; }
-__device__ __forceinline__ int* cnt3_of(const FArgs& a) { return cnt2_of(a) + a.Gmax * a.NB2; }
 
 // ---- device-coherent (cross-XCD) accesses
-__device__ __forceinline__ int ld_acquire(const int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ uint64_t ld_dev64(const void* p) { return __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_dev64(void* p, uint64_t v) { __hip_atomic_store((uint64_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ uint32_t ld_dev32(const void* p) { return __hip_atomic_load((const uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_dev32(void* p, uint32_t v) { __hip_atomic_store((uint32_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-// ---- XCD-local accesses: an ordinary store reaches the XCD's L2 (the L1 is write-through); a load with sc0 misses the
-// L1 and reads that L2.  Eight 8-byte loads are issued together and waited for once.
-__device__ __forceinline__ void ld_l2x8(const void* const (&p)[8], uint64_t (&o)[8])
+// ---- XCD-local accesses: an ordinary store reaches the XCD's L2 (the L1 is write-through).  A load, whatever its cache
+// bits short of device scope, may be served from the CU's L1 once the line is there, so a consumer that polls would spin
+// on a stale line: it takes the word with an exchange instead, which executes in the L2 and leaves EMPTY behind.
+__device__ __forceinline__ uint64_t swap_l2(float* p)
 {
-    asm volatile(
-        "global_load_dwordx2 %0, %8, off sc0\n\tglobal_load_dwordx2 %1, %9, off sc0\n\tglobal_load_dwordx2 %2, %10, off sc0\n\t"
-        "global_load_dwordx2 %3, %11, off sc0\n\tglobal_load_dwordx2 %4, %12, off sc0\n\tglobal_load_dwordx2 %5, %13, off sc0\n\t"
-        "global_load_dwordx2 %6, %14, off sc0\n\tglobal_load_dwordx2 %7, %15, off sc0\n\ts_waitcnt vmcnt(0)"
-        : "=&v"(o[0]), "=&v"(o[1]), "=&v"(o[2]), "=&v"(o[3]), "=&v"(o[4]), "=&v"(o[5]), "=&v"(o[6]), "=&v"(o[7])
-        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
-        : "memory");
+    return __hip_atomic_exchange((uint64_t*)p, EMPTY2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
-// up to 8 pairs of floats from 8 addresses (slots >= n repeat slot 0 and are ignored), XCD-local or device-coherent
-__device__ __forceinline__ void gather8(bool local, const float* const (&p)[8], int n, float (&lo)[8], float (&hi)[8])
+__device__ __forceinline__ uint32_t fbits(float v) { const uint32_t u = __float_as_uint(v); return u == EMPTY ? 0x7fc00000u : u; }
+// producer side: two adjacent words
+__device__ __forceinline__ void put2(bool local, float* p, float v0, float v1)
+{
+    const uint64_t u = (uint64_t)fbits(v0) | ((uint64_t)fbits(v1) << 32);
+    if (local) *(uint64_t*)p = u; else st_dev64(p, u);
+}
+// consumer side, whole wave: waits until the n (<= 8) word pairs at p[] all hold data, returns them and leaves the words
+// EMPTY again.  Slots >= n are ignored.  The outcome is the same for every lane; false = the wait expired.
+__device__ __forceinline__ bool take8(bool local, float* const (&p)[8], int n, float (&lo)[8], float (&hi)[8])
 {
     uint64_t o[8];
-    if (local) {
-        const void* q[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[i] = i < n ? p[i] : p[0];
-        ld_l2x8(q, o);
-    } else {
+    for (int i = 0; i < 8; ++i) o[i] = i < n ? EMPTY2 : 0;
+    int spins = 0;
+    for (;;) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] = i < n ? ld_dev64(p[i]) : 0;
+        for (int i = 0; i < 8; ++i)
+            if (i < n && o[i] == EMPTY2) o[i] = local ? swap_l2(p[i]) : ld_dev64(p[i]);
+        bool ok = true;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ok = ok && o[i] != EMPTY2;
+        if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+        if (++spins >= SPIN_MAX) return false;
+        __builtin_amdgcn_s_sleep(1);
+    }
+    if (!local) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (i < n) st_dev64(p[i], EMPTY2);
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) { lo[i] = __uint_as_float((uint32_t)o[i]); hi[i] = __uint_as_float((uint32_t)(o[i] >> 32)); }
-}
-__device__ __forceinline__ void put2(bool local, float* p, float v0, float v1)
-{
-    const uint64_t u = (uint64_t)__float_as_uint(v0) | ((uint64_t)__float_as_uint(v1) << 32);
-    if (local) *(uint64_t*)p = u; else st_dev64(p, u);
-}
-// all of this wave's stores have been acknowledged (then __syncthreads() covers the block)
-__device__ __forceinline__ void stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-// counter bump that publishes the block's data: one thread, after stores_done() + __syncthreads() of every wave
-__device__ __forceinline__ int bump(bool local, int* p)
-{
-    return local ? __hip_atomic_fetch_add(p, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)     // executes in the XCD's L2
-                 : __hip_atomic_fetch_add(p, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
 }
 
 struct Group { int e, n; };
 // item g of the call: expert and its pair rows (ascending), or n = 0 when the call has fewer items.  All threads call.
+// Leaves every pair's expert in sidx[] when R > 1.
 __device__ __forceinline__ Group find_item(const FArgs& a, int g, int* sidx, unsigned char* isf, int* rows, int* misc)
 {
     const int P = a.P, tid = threadIdx.x;
@@ -150,7 +158,7 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
 {
     __shared__ __align__(16) uint16_t xs[MR][KTB * 16];   // this block's K slice of the transformed activations (fp16)
     __shared__ float red[FW][MR][128];
-    __shared__ int sidx[PF_MAX], rows[RF_MAX], misc[4];
+    __shared__ int sidx[PF_MAX], rows[RF_MAX], comb[RF_MAX], misc[4];
     __shared__ unsigned char isf[PF_MAX];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bid = blockIdx.x;
@@ -170,46 +178,63 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
             K = c.I; N = c.H;
         }
     }
+    if (isA) __builtin_amdgcn_s_setprio(2);               // stage 1 is the critical path: its waves issue first
     TRACE(0);
+    if (tid == 0) misc[2] = 1;
     Group grp{0, 0};
     if (g >= 0) grp = find_item(a, g, sidx, isf, rows, misc);
     TRACE(1);
-    bool alive = grp.n > 0;
-    if (alive) {
+    if (grp.n > 0) {
         const int Kt = K / 16, Nt = N / 16;
         const int kt0 = s * KTB, kt1 = min(Kt, kt0 + KTB), nkt = kt1 - kt0;
         const int nblk = (nkt + 7) / 8;                   // 128-blocks of K in this slice
         const uint32_t* tr = (const uint32_t*)a.tab[(int64_t)(isA ? t : 2) * c.E + grp.e];
-        // ---- issue this wave's tile loads: k-tiles kt0 + wave + FW i
-        uint4 wr[TW];
-#pragma unroll
-        for (int i = 0; i < TW; ++i) {
-            const int kt = kt0 + wave + FW * i;
-            wr[i] = make_uint4(0u, 0u, 0u, 0u);
-            if (kt < kt1) wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
-        }
-        TRACE(2);
         const int src = tile_prev_lane(lane);
         const int ncol = nb * 128 + 2 * lane;             // this lane's two columns in the finishing steps
+        const int j8 = lane >> 3, m8 = lane & 7;
         float acc[MR][2];
 #pragma unroll
         for (int r = 0; r < MR; ++r) { acc[r][0] = 0.f; acc[r][1] = 0.f; }
         if (isA) {
-            // ---- scales of the finishing step, fetched early (any block of the group may be its last)
+            const bool finisher = t == 1 && s == a.S1 - 1;
+            // ---- the slice of x and its sign vector first (the transform overlaps the weight stream), then the tiles
             const uint16_t* suh = (const uint16_t*)a.tab[(int64_t)(3 + t) * c.E + grp.e];
-            const uint16_t* svg = (const uint16_t*)a.tab[(int64_t)6 * c.E + grp.e];
-            const uint16_t* svu = (const uint16_t*)a.tab[(int64_t)7 * c.E + grp.e];
-            const uint16_t* sud = (const uint16_t*)a.tab[(int64_t)5 * c.E + grp.e];
-            const float sg0 = f16_bits_to_f32(svg[ncol]), sg1 = f16_bits_to_f32(svg[ncol + 1]);
-            const float su0 = f16_bits_to_f32(svu[ncol]), su1 = f16_bits_to_f32(svu[ncol + 1]);
-            const float sd0 = f16_bits_to_f32(sud[ncol]), sd1 = f16_bits_to_f32(sud[ncol + 1]);
-            // ---- transform the slice of x into LDS: wave per (row, 128-block)
-            for (int u = wave; u < grp.n * nblk; u += FW) {
-                const int r = u / nblk, kb = u % nblk;
-                const int k = kt0 * 16 + kb * 128 + 2 * lane;
+            float xv0 = 0.f, xv1 = 0.f;
+            const int unit0 = wave;                       // first (row, 128-block) unit of this wave
+            if (unit0 < grp.n * nblk) {
+                const int r = unit0 / nblk, kb = unit0 % nblk, k = kt0 * 16 + kb * 128 + 2 * lane;
                 const int64_t srow = rows[r] / c.topk;
-                float v0 = exl3_ld_x(a.x, c.xtype, srow * a.ldx + k) * f16_bits_to_f32(suh[k]);
-                float v1 = exl3_ld_x(a.x, c.xtype, srow * a.ldx + k + 1) * f16_bits_to_f32(suh[k + 1]);
+                xv0 = exl3_ld_x(a.x, c.xtype, srow * a.ldx + k) * f16_bits_to_f32(suh[k]);
+                xv1 = exl3_ld_x(a.x, c.xtype, srow * a.ldx + k + 1) * f16_bits_to_f32(suh[k + 1]);
+            }
+            uint4 wr[TW];
+#pragma unroll
+            for (int i = 0; i < TW; ++i) {
+                const int kt = kt0 + wave + FW * i;
+                wr[i] = make_uint4(0u, 0u, 0u, 0u);
+                if (kt < kt1) wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
+            }
+            TRACE(2);
+            // ---- scales of the finishing step (the finisher only)
+            float sg0 = 0.f, sg1 = 0.f, su0 = 0.f, su1 = 0.f, sd0 = 0.f, sd1 = 0.f;
+            if (finisher) {
+                const uint16_t* svg = (const uint16_t*)a.tab[(int64_t)6 * c.E + grp.e];
+                const uint16_t* svu = (const uint16_t*)a.tab[(int64_t)7 * c.E + grp.e];
+                const uint16_t* sud = (const uint16_t*)a.tab[(int64_t)5 * c.E + grp.e];
+                sg0 = f16_bits_to_f32(svg[ncol]); sg1 = f16_bits_to_f32(svg[ncol + 1]);
+                su0 = f16_bits_to_f32(svu[ncol]); su1 = f16_bits_to_f32(svu[ncol + 1]);
+                sd0 = f16_bits_to_f32(sud[ncol]); sd1 = f16_bits_to_f32(sud[ncol + 1]);
+            }
+            // ---- transform the slice of x into LDS: wave per (row, 128-block)
+            for (int u = unit0; u < grp.n * nblk; u += FW) {
+                const int r = u / nblk, kb = u % nblk;
+                float v0 = xv0, v1 = xv1;
+                if (u != unit0) {
+                    const int k = kt0 * 16 + kb * 128 + 2 * lane;
+                    const int64_t srow = rows[r] / c.topk;
+                    v0 = exl3_ld_x(a.x, c.xtype, srow * a.ldx + k) * f16_bits_to_f32(suh[k]);
+                    v1 = exl3_ld_x(a.x, c.xtype, srow * a.ldx + k + 1) * f16_bits_to_f32(suh[k + 1]);
+                }
                 fwht128(v0, v1, lane);
                 *(uint32_t*)&xs[r][kb * 128 + 2 * lane] = (uint32_t)f32_to_f16_bits(v0) | ((uint32_t)f32_to_f16_bits(v1) << 16);
             }
@@ -229,76 +254,115 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
                 }
             }
             TRACE(5);
-            // ---- sum the waves in wave order, publish the partial of this (matrix, K slice) inside the XCD
-            const int j = lane >> 3, m = lane & 7;
+            // ---- sum the waves in wave order; every block but the finisher hands its partial over inside the XCD
 #pragma unroll
-            for (int r = 0; r < MR; ++r) { red[wave][r][16 * j + m] = acc[r][0]; red[wave][r][16 * j + m + 8] = acc[r][1]; }
+            for (int r = 0; r < MR; ++r) { red[wave][r][16 * j8 + m8] = acc[r][0]; red[wave][r][16 * j8 + m8 + 8] = acc[r][1]; }
             __syncthreads();
-            float* part = a.part1 + ((int64_t)(s * 2 + t) * a.P) * N;
-            for (int i = tid; i < grp.n * 64; i += 64 * FW) {
-                const int r = i >> 6, col = (i & 63) * 2;
-                float v0 = red[0][r][col], v1 = red[0][r][col + 1];
+            if (!finisher) {
+                float* part = a.part1 + ((int64_t)(s * 2 + t) * a.P) * N;
+                for (int i = tid; i < grp.n * 64; i += 64 * FW) {
+                    const int r = i >> 6, col = (i & 63) * 2;
+                    float v0 = red[0][r][col], v1 = red[0][r][col + 1];
 #pragma unroll
-                for (int w = 1; w < FW; ++w) { v0 += red[w][r][col]; v1 += red[w][r][col + 1]; }
-                put2(local, &part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
-            }
-            stores_done();
-            __syncthreads();
-            if (tid == 0) misc[3] = bump(local, cnt1_of(a) + g * a.NB1 + nb) == 2 * a.S1 - 1;
-            __syncthreads();
-            TRACE(6);
-            if (misc[3]) {
-                // ---- last block of the group: finish gate and up, activation, down input transform -> xh2 (device-coherent)
+                    for (int w = 1; w < FW; ++w) { v0 += red[w][r][col]; v1 += red[w][r][col + 1]; }
+                    put2(local, &part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
+                }
+                TRACE(6);
+            } else {
+                // ---- finisher: gate and up sums in slice order, Hadamard, svh, activation, down input transform -> xh2
+                bool good = true;
                 for (int r = wave; r < grp.n; r += FW) {
                     float gl[8], gh[8], ul[8], uh[8];
-                    const float* pg[8]; const float* pu[8];
+                    float* pg[8]; float* pu[8];
 #pragma unroll
                     for (int ss = 0; ss < 8; ++ss) {
                         const int s2 = ss < a.S1 ? ss : 0;
                         pg[ss] = a.part1 + ((int64_t)(s2 * 2 + 0) * a.P + rows[r]) * c.I + ncol;
                         pu[ss] = a.part1 + ((int64_t)(s2 * 2 + 1) * a.P + rows[r]) * c.I + ncol;
                     }
-                    gather8(local, pg, a.S1, gl, gh);
-                    gather8(local, pu, a.S1, ul, uh);
+                    good = take8(local, pg, a.S1, gl, gh) && good;
+                    if (a.S1 > 1) good = take8(local, pu, a.S1 - 1, ul, uh) && good;
                     float g0 = 0.f, g1 = 0.f, u0 = 0.f, u1 = 0.f;
 #pragma unroll
-                    for (int ss = 0; ss < 8; ++ss) if (ss < a.S1) { g0 += gl[ss]; g1 += gh[ss]; u0 += ul[ss]; u1 += uh[ss]; }
+                    for (int ss = 0; ss < 8; ++ss) if (ss < a.S1) { g0 += gl[ss]; g1 += gh[ss]; }
+#pragma unroll
+                    for (int ss = 0; ss < 8; ++ss) if (ss < a.S1 - 1) { u0 += ul[ss]; u1 += uh[ss]; }
+                    float o0 = red[0][r][2 * lane], o1 = red[0][r][2 * lane + 1];      // this block's own slice of up, last in order
+#pragma unroll
+                    for (int w = 1; w < FW; ++w) { o0 += red[w][r][2 * lane]; o1 += red[w][r][2 * lane + 1]; }
+                    u0 += o0; u1 += o1;
                     fwht128(g0, g1, lane);
                     fwht128(u0, u1, lane);
                     float v0 = exl3_act(c.act, g0 * sg0, u0 * su0) * sd0;
                     float v1 = exl3_act(c.act, g1 * sg1, u1 * su1) * sd1;
                     fwht128(v0, v1, lane);
-                    st_dev32(a.xh2 + (int64_t)rows[r] * c.I + ncol, (uint32_t)f32_to_f16_bits(v0) | ((uint32_t)f32_to_f16_bits(v1) << 16));
+                    uint32_t pk = (uint32_t)f32_to_f16_bits(v0) | ((uint32_t)f32_to_f16_bits(v1) << 16);
+                    if (pk == EMPTY) pk = 0x7e007e00u;
+                    if (good)
+                        for (int q = 0; q < a.NB2; ++q) st_dev32(a.xh2 + ((int64_t)q * a.P + rows[r]) * (c.I / 2) + (ncol >> 1), pk);
                 }
-                stores_done();
-                __syncthreads();
-                if (tid == 0) bump(false, ready_of(a) + g);
+                TRACE(6);
+                if (!good && lane == 0) atomicExch(a.err, 1);
             }
         } else {
-            // ---- decode first and fetch the finishing scales (independent of stage 1), then wait for the item's xh2
+            // ---- issue the tile loads, decode and fetch the finishing scales (independent of stage 1), then take xh2
+            uint4 wr[TW];
+#pragma unroll
+            for (int i = 0; i < TW; ++i) {
+                const int kt = kt0 + wave + FW * i;
+                wr[i] = make_uint4(0u, 0u, 0u, 0u);
+                if (kt < kt1) wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
+            }
+            TRACE(2);
+            const bool finisher = s == a.S2 - 1;
+            const uint16_t* svd = (const uint16_t*)a.tab[(int64_t)8 * c.E + grp.e];
+            const float svd0 = f16_bits_to_f32(svd[ncol]), svd1 = f16_bits_to_f32(svd[ncol + 1]);
+            // rows of this item whose weighted sum this block does: those whose other experts all belong to earlier items
+            if (finisher) {
+                if (a.R == 1) { if (tid == 0) comb[0] = g == a.P - 1; }
+                else {
+                    if (tid < grp.n) comb[tid] = 1;
+                    __syncthreads();
+                    const int fo = rows[0];               // first pair of this item's expert
+                    for (int u = tid; u < grp.n * c.topk; u += 64 * FW) {
+                        const int i = u / c.topk, k = u % c.topk, e = sidx[(rows[i] / c.topk) * c.topk + k];
+                        bool seen = false;
+                        for (int q = 0; q <= fo; ++q) seen |= sidx[q] == e;
+                        if (!seen) comb[i] = 0;
+                    }
+                }
+            }
             h2 wd[TW][4][4];
 #pragma unroll
             for (int i = 0; i < TW; ++i) decode_tile32<CBK>(wr[i], __shfl(wr[i].w, src, 64), wd[i]);
-            const uint16_t* svd = (const uint16_t*)a.tab[(int64_t)8 * c.E + grp.e];
-            const float svd0 = f16_bits_to_f32(svd[ncol]), svd1 = f16_bits_to_f32(svd[ncol + 1]);
             asm volatile("" :: "v"(svd0), "v"(svd1));
             TRACE(3);
-            if (tid == 0) {
-                const int* rdy = ready_of(a) + g;
+            __builtin_amdgcn_s_setprio(3);
+            uint32_t* xc = a.xh2 + ((int64_t)nb * a.P) * (c.I / 2) + kt0 * 8;         // this column block's copy, this K slice
+            // cheap wait first: one word per 128-block of the slice (the finishers' last lanes), then every word
+            if (wave == 0) {
                 int spins = 0;
-                while (ld_acquire(rdy) < a.NB1 && spins < SPIN_MAX) { __builtin_amdgcn_s_sleep(2); ++spins; }
-                misc[2] = spins < SPIN_MAX;
-                if (spins >= SPIN_MAX) atomicExch(&a.cnt[1], 1);
+                for (;;) {
+                    const uint32_t v = lane < nblk ? ld_dev32(xc + (int64_t)rows[0] * (c.I / 2) + lane * 64 + 63) : 0u;
+                    if (__builtin_amdgcn_ballot_w64(v == EMPTY) == 0 || ++spins >= SPIN_MAX) break;
+                    __builtin_amdgcn_s_sleep(2);
+                }
             }
             __syncthreads();
+            bool good = true;
+            for (int u = tid; u < grp.n * (nkt * 8); u += 64 * FW) {                  // 2 fp16 per thread-step
+                const int r = u / (nkt * 8), q = u % (nkt * 8);
+                uint32_t* p = xc + (int64_t)rows[r] * (c.I / 2) + q;
+                uint32_t v;
+                int spins = 0;
+                while ((v = ld_dev32(p)) == EMPTY && ++spins < SPIN_MAX) __builtin_amdgcn_s_sleep(1);
+                if (v == EMPTY) good = false; else st_dev32(p, EMPTY);
+                *(uint32_t*)&xs[r][q * 2] = v;
+            }
+            if (!good) misc[2] = 0;
+            __syncthreads();
             TRACE(4);
-            alive = misc[2] != 0;
-            if (alive) {
-                for (int u = tid; u < grp.n * (nkt * 8); u += 64 * FW) {      // 2 fp16 per thread-step
-                    const int r = u / (nkt * 8), q = u % (nkt * 8);
-                    *(uint32_t*)&xs[r][q * 2] = ld_dev32((const uint32_t*)(a.xh2 + (int64_t)rows[r] * c.I + kt0 * 16) + q);
-                }
-                __syncthreads();
+            if (misc[2]) {
 #pragma unroll
                 for (int i = 0; i < TW; ++i) {
                     const int kt = kt0 + wave + FW * i;
@@ -311,12 +375,10 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
                     }
                 }
                 TRACE(5);
-                const int j = lane >> 3, m = lane & 7;
 #pragma unroll
-                for (int r = 0; r < MR; ++r) { red[wave][r][16 * j + m] = acc[r][0]; red[wave][r][16 * j + m + 8] = acc[r][1]; }
+                for (int r = 0; r < MR; ++r) { red[wave][r][16 * j8 + m8] = acc[r][0]; red[wave][r][16 * j8 + m8 + 8] = acc[r][1]; }
                 __syncthreads();
-                bool last = true;
-                if (a.S2 > 1) {
+                if (!finisher) {
                     float* part = a.part2 + ((int64_t)s * a.P) * N;
                     for (int i = tid; i < grp.n * 64; i += 64 * FW) {
                         const int r = i >> 6, col = (i & 63) * 2;
@@ -325,51 +387,41 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
                         for (int w = 1; w < FW; ++w) { v0 += red[w][r][col]; v1 += red[w][r][col + 1]; }
                         put2(local, &part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
                     }
-                    stores_done();
-                    __syncthreads();
-                    if (tid == 0) misc[3] = bump(local, cnt2_of(a) + g * a.NB2 + nb) == a.S2 - 1;
-                    __syncthreads();
-                    last = misc[3] != 0;
-                }
-                TRACE(6);
-                if (last) {
-                    // ---- finish the down product: yd[pair] = had128(sum of slices) * svh; wave per row
+                    TRACE(6);
+                } else {
+                    // ---- finish the down product: yd[pair] = had128(sum of slices in order) * svh; wave per row
+                    bool ok = true;
                     for (int r = wave; r < grp.n; r += FW) {
                         float v0 = 0.f, v1 = 0.f;
                         if (a.S2 > 1) {
                             float pl[8], ph[8];
-                            const float* pp[8];
+                            float* pp[8];
 #pragma unroll
-                            for (int ss = 0; ss < 8; ++ss) pp[ss] = a.part2 + ((int64_t)(ss < a.S2 ? ss : 0) * a.P + rows[r]) * c.H + ncol;
-                            gather8(local, pp, a.S2, pl, ph);
+                            for (int ss = 0; ss < 8; ++ss) pp[ss] = a.part2 + ((int64_t)(ss < a.S2 - 1 ? ss : 0) * a.P + rows[r]) * c.H + ncol;
+                            ok = take8(local, pp, a.S2 - 1, pl, ph) && ok;
 #pragma unroll
-                            for (int ss = 0; ss < 8; ++ss) if (ss < a.S2) { v0 += pl[ss]; v1 += ph[ss]; }
-                        } else {
-#pragma unroll
-                            for (int w = 0; w < FW; ++w) { v0 += red[w][r][2 * lane]; v1 += red[w][r][2 * lane + 1]; }
+                            for (int ss = 0; ss < 8; ++ss) if (ss < a.S2 - 1) { v0 += pl[ss]; v1 += ph[ss]; }
                         }
+                        float o0 = red[0][r][2 * lane], o1 = red[0][r][2 * lane + 1];
+#pragma unroll
+                        for (int w = 1; w < FW; ++w) { o0 += red[w][r][2 * lane]; o1 += red[w][r][2 * lane + 1]; }
+                        v0 += o0; v1 += o1;
                         fwht128(v0, v1, lane);
-                        put2(local, a.yd + (int64_t)rows[r] * c.H + ncol, v0 * svd0, v1 * svd1);
+                        if (ok) put2(local, a.yd + (int64_t)rows[r] * c.H + ncol, v0 * svd0, v1 * svd1);
                     }
-                    stores_done();
-                    __syncthreads();
-                    // ---- rows whose last expert just arrived: weighted slot-order sum of this column block
-                    if (tid < grp.n) {
-                        const int r = rows[tid] / c.topk;
-                        sidx[tid] = bump(local, cnt3_of(a) + r * a.NB2 + nb) == c.topk - 1 ? r : -1;
-                    }
-                    __syncthreads();
+                    TRACE(6);
+                    // ---- rows this block sums: every expert's output of the row, in slot order, weighted
                     for (int i = wave; i < grp.n; i += FW) {
-                        const int r = sidx[i];
-                        if (r < 0) continue;
+                        if (!comb[i]) continue;
+                        const int r = rows[i] / c.topk;
                         float a0 = 0.f, a1 = 0.f;
                         for (int k0 = 0; k0 < c.topk; k0 += 8) {                // 8 experts' outputs requested together
                             float yl[8], yh[8];
-                            const float* py[8];
+                            float* py[8];
                             const int nk = min(8, c.topk - k0);
 #pragma unroll
                             for (int k = 0; k < 8; ++k) py[k] = a.yd + (int64_t)(r * c.topk + k0 + (k < nk ? k : 0)) * c.H + ncol;
-                            gather8(local, py, nk, yl, yh);
+                            ok = take8(local, py, nk, yl, yh) && ok;
 #pragma unroll
                             for (int k = 0; k < 8; ++k)
                                 if (k < nk) {
@@ -378,33 +430,24 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
                                 }
                         }
                         const float b0 = a.add ? a.add[(int64_t)r * c.H + ncol] : 0.f, b1 = a.add ? a.add[(int64_t)r * c.H + ncol + 1] : 0.f;
-                        a.out[(int64_t)r * c.H + ncol] = b0 + a0;
-                        a.out[(int64_t)r * c.H + ncol + 1] = b1 + a1;
+                        if (ok) {
+                            a.out[(int64_t)r * c.H + ncol] = b0 + a0;
+                            a.out[(int64_t)r * c.H + ncol + 1] = b1 + a1;
+                        }
                     }
+                    if (!ok && lane == 0) atomicExch(a.err, 1);
                 }
-            }
+            } else if (tid == 0) atomicExch(a.err, 1);
         }
     }
-    // ---- every block ends here: the last block of an XCD reports to the device-wide counter, the last of those clears
-    // the counters for the next call (nothing else is running then)
-    __syncthreads();
     TRACE(7);
-    if (tid == 0) {
-        const int xcd = bid % NXCD, mine = ((int)gridDim.x - xcd + NXCD - 1) / NXCD;   // blocks with this id % 8
-        bool fin = false;
-        if (bump(local, a.cnt + 2 + xcd) == mine - 1) fin = bump(false, a.cnt) == NXCD - 1;
-        misc[0] = fin;
-    }
-    __syncthreads();
-    if (misc[0]) {
-        for (int i = tid; i < a.ncnt; i += 64 * FW) if (i != 1) a.cnt[i] = 0;
-    }
 }
 
-__global__ void zero_kernel(int* p, int n)
+// every exchanged word EMPTY, the error flag clear
+__global__ void fill_kernel(uint32_t* p, int64_t n)
 {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = i < HEAD / 4 ? 0u : EMPTY;
 }
 // the XCD a workgroup runs on (XCC_ID, hardware register 20)
 __global__ void xcd_probe_kernel(int* out)
@@ -412,7 +455,7 @@ __global__ void xcd_probe_kernel(int* out)
     if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((31 << 11) | 20) & 0xf;
 }
 
-struct FPlan { int P, Gmax, S1, S2, NB1, NB2, nA, nB, ncnt, bpgA, bpgB; size_t cnt, part1, xh2, part2, yd, total; };
+struct FPlan { int P, Gmax, S1, S2, NB1, NB2, nA, nB, bpgA, bpgB; size_t part1, xh2, part2, yd, total; };
 FPlan fplan(const Exl3Cfg& c, int R)
 {
     FPlan p;
@@ -425,13 +468,11 @@ FPlan fplan(const Exl3Cfg& c, int R)
     const int QA = (p.Gmax * p.NB1 + NXCD - 1) / NXCD * NXCD, QB = (p.NB2 + NXCD - 1) / NXCD * NXCD;   // groups, padded to the XCD count
     p.nA = QA * p.bpgA;
     p.nB = QB * p.bpgB;
-    p.ncnt = 2 + NXCD + p.Gmax * p.NB1 + p.Gmax + p.Gmax * p.NB2 + R * p.NB2;
-    size_t o = 0;
+    size_t o = HEAD;
     auto take = [&](size_t n) { const size_t q = o; o += align256(n); return q; };
-    p.cnt = take(4 * (size_t)p.ncnt);
     p.part1 = take(4 * (size_t)p.S1 * 2 * p.P * c.I);
-    p.xh2 = take(2 * (size_t)p.P * c.I);
-    p.part2 = take(4 * (size_t)p.S2 * p.P * c.H);
+    p.xh2 = take(4 * (size_t)p.NB2 * p.P * (c.I / 2));
+    p.part2 = take(p.S2 > 1 ? 4 * (size_t)p.S2 * p.P * c.H : 0);
     p.yd = take(4 * (size_t)p.P * c.H);
     p.total = o;
     return p;
@@ -477,6 +518,14 @@ int exl3_xcd_probe()
     return g_xcd_local = ok ? 1 : 0;
 }
 
+// Every exchanged word of a workspace EMPTY and its error flag clear (any size: the whole buffer is filled).
+int exl3_fused_ws_prepare(void* ws, size_t bytes, hipStream_t st)
+{
+    const int64_t n = (int64_t)(bytes / 4);
+    if (n > 0) fill_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((uint32_t*)ws, n);
+    return launch_status();
+}
+
 int exl3_fused_launch(const Exl3Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
                       int clean, hipStream_t st)
 {
@@ -484,13 +533,16 @@ int exl3_fused_launch(const Exl3Cfg& c, const void* x, int64_t ldx, int R, const
     char* b = (char*)ws;
     FArgs a;
     a.x = x; a.ldx = ldx; a.idx = idx; a.w = w; a.tab = (const uint64_t*)tab; a.add = (const float*)add; a.out = (float*)out;
-    a.cnt = (int*)(b + p.cnt); a.part1 = (float*)(b + p.part1); a.xh2 = (uint16_t*)(b + p.xh2); a.part2 = (float*)(b + p.part2); a.yd = (float*)(b + p.yd);
-    a.R = R; a.P = p.P; a.Gmax = p.Gmax; a.S1 = p.S1; a.S2 = p.S2; a.NB1 = p.NB1; a.NB2 = p.NB2; a.nA = p.nA; a.nB = p.nB; a.ncnt = p.ncnt;
+    a.err = (int*)b; a.part1 = (float*)(b + p.part1); a.xh2 = (uint32_t*)(b + p.xh2); a.part2 = (float*)(b + p.part2); a.yd = (float*)(b + p.yd);
+    a.R = R; a.P = p.P; a.Gmax = p.Gmax; a.S1 = p.S1; a.S2 = p.S2; a.NB1 = p.NB1; a.NB2 = p.NB2; a.nA = p.nA; a.nB = p.nB;
     a.bpgA = p.bpgA; a.bpgB = p.bpgB;
     a.local = g_xcd_local == 1;
     a.c = c;
     a.trace = g_trace;
-    if (!clean) zero_kernel<<<(p.ncnt + 255) / 256, 256, 0, st>>>(a.cnt, p.ncnt);
+    if (!clean) {
+        const int rc = exl3_fused_ws_prepare(ws, p.total, st);
+        if (rc) return rc;
+    }
     if (c.cbk == CB_MCG) launch<CB_MCG>(a, R, st);
     else launch<CB_MUL1>(a, R, st);
     return launch_status();
