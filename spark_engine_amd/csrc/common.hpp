@@ -84,18 +84,44 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
+// The value lane ^ M holds, without LDS traffic: DPP quad permutes and row mirrors inside a row of 16 lanes (xor 4 = reverse
+// the quad then mirror the half row, xor 8 = mirror the half row then the row), the gfx950 row / half-wave swaps beyond.
+template <int CTRL> __device__ __forceinline__ float dpp_mov_f32(float v)
+{
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xf, 0xf, false));
+}
+template <int M> __device__ __forceinline__ float lane_xor(float v, int lane)
+{
+    static_assert(M == 1 || M == 2 || M == 4 || M == 8 || M == 16 || M == 32, "one bit");
+    if constexpr (M == 1) return dpp_mov_f32<0xB1>(v);                        // quad_perm [1,0,3,2]
+    else if constexpr (M == 2) return dpp_mov_f32<0x4E>(v);                   // quad_perm [2,3,0,1]
+    else if constexpr (M == 4) return dpp_mov_f32<0x141>(dpp_mov_f32<0x1B>(v));   // quad_perm [3,2,1,0], row_half_mirror
+    else if constexpr (M == 8) return dpp_mov_f32<0x140>(dpp_mov_f32<0x141>(v));  // row_half_mirror, row_mirror
+    else if constexpr (M == 16) {
+        // vdst' = rows (0, 0, 2, 2) of v, src' = rows (1, 1, 3, 3)
+        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        return __uint_as_float((lane & 16) ? r[0] : r[1]);
+    } else {
+        // vdst' = the lower half twice, src' = the upper half twice
+        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        return __uint_as_float((lane & 32) ? r[0] : r[1]);
+    }
+}
+template <int M> __device__ __forceinline__ void fwht_stage(float& v0, float& v1, int lane)
+{
+    // (a + b, a - b) with the lower lane holding a: upper lanes negate their own value first, then both add
+    const uint32_t sign = (lane & M) ? 0x80000000u : 0u;
+    const float o0 = lane_xor<M>(v0, lane), o1 = lane_xor<M>(v1, lane);
+    v0 = o0 + __uint_as_float(__float_as_uint(v0) ^ sign);
+    v1 = o1 + __uint_as_float(__float_as_uint(v1) ^ sign);
+}
 // 128-point normalized Walsh-Hadamard over values held 2 per lane (lane l: elements 2l, 2l+1), binary32, butterflies
 // h = 1, 2, ..., 64 with (a + b, a - b), lower index first, then one multiply: the operation order of a serial FWHT.
 __device__ __forceinline__ void fwht128(float& v0, float& v1, int lane)
 {
     { const float a = v0 + v1, b = v0 - v1; v0 = a; v1 = b; }
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) {
-        const bool upper = lane & m;
-        const float o0 = __shfl_xor(v0, m, 64), o1 = __shfl_xor(v1, m, 64);
-        v0 = upper ? o0 - v0 : v0 + o0;
-        v1 = upper ? o1 - v1 : v1 + o1;
-    }
+    fwht_stage<1>(v0, v1, lane); fwht_stage<2>(v0, v1, lane); fwht_stage<4>(v0, v1, lane);
+    fwht_stage<8>(v0, v1, lane); fwht_stage<16>(v0, v1, lane); fwht_stage<32>(v0, v1, lane);
     v0 *= 0.08838834764831845f;
     v1 *= 0.08838834764831845f;
 }

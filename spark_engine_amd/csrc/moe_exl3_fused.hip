@@ -41,8 +41,8 @@ long long* g_trace = nullptr;
 #define TRACE(i) do { if (a.trace && tid == 0) a.trace[(int64_t)bid * 8 + (i)] = wall_clock64(); } while (0)
 
 constexpr int FW = 4;                 // waves per block
-constexpr int TW = 8;                 // k-tiles per wave (all loaded up front)
-constexpr int KTB = FW * TW;          // k-tiles per block = K slice of 512
+constexpr int TWB = 8;                // k-tiles per wave of a stage-2 block (all loaded up front): K slice of 512
+constexpr int TWMAX = 8;              // most k-tiles per wave of a stage-1 block (4 or 8, chosen per shape)
 constexpr int PF_MAX = 256, RF_MAX = 16;
 constexpr int SPIN_MAX = 200000;
 constexpr int SMAX = 8;               // K slices per product (K <= 4096)
@@ -58,7 +58,7 @@ struct FArgs {
     float* part2;                     // [S2][P][H] down partial sums per K slice (S2 > 1 only)
     float* yd;                        // [P][H] per-pair expert outputs
     int* err;
-    int R, P, Gmax, S1, S2, NB1, NB2, nA, nB, bpgA, bpgB, local;
+    int R, P, Gmax, S1, S2, NB1, NB2, nA, nB, bpgA, bpgB, local;     // S1 / S2 = K slices of stage 1 / 2
     Exl3Cfg c;
     long long* trace;                 // optional per-block timestamps (diagnostics), 8 per block
 };
@@ -68,47 +68,59 @@ __device__ __forceinline__ uint64_t ld_dev64(const void* p) { return __hip_atomi
 __device__ __forceinline__ void st_dev64(void* p, uint64_t v) { __hip_atomic_store((uint64_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ uint32_t ld_dev32(const void* p) { return __hip_atomic_load((const uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_dev32(void* p, uint32_t v) { __hip_atomic_store((uint32_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-// ---- XCD-local accesses: an ordinary store reaches the XCD's L2 (the L1 is write-through).  A load, whatever its cache
-// bits short of device scope, may be served from the CU's L1 once the line is there, so a consumer that polls would spin
-// on a stale line: it takes the word with an exchange instead, which executes in the L2 and leaves EMPTY behind.
-__device__ __forceinline__ uint64_t swap_l2(float* p)
+// ---- XCD-local accesses: an ordinary store reaches the XCD's L2 (the L1 is write-through).  An ordinary or sc0 load may be
+// served from the CU's L1 once the line is there, so a consumer that polls with it spins on a stale line (measured); a
+// non-temporal load is not kept in the L1 and reads the L2 every time (measured: 0.3 us from store to observation).
+__device__ __forceinline__ uint64_t ld_l2(const float* p)
 {
-    return __hip_atomic_exchange((uint64_t*)p, EMPTY2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    return __builtin_nontemporal_load((const __attribute__((address_space(1))) uint64_t*)(uintptr_t)p);
 }
 __device__ __forceinline__ uint32_t fbits(float v) { const uint32_t u = __float_as_uint(v); return u == EMPTY ? 0x7fc00000u : u; }
 // producer side: two adjacent words
-__device__ __forceinline__ void put2(bool local, float* p, float v0, float v1)
+template <bool local> __device__ __forceinline__ void put2(float* p, float v0, float v1)
 {
     const uint64_t u = (uint64_t)fbits(v0) | ((uint64_t)fbits(v1) << 32);
     if (local) *(uint64_t*)p = u; else st_dev64(p, u);
 }
-// consumer side, whole wave: waits until the n (<= 8) word pairs at p[] all hold data, returns them and leaves the words
-// EMPTY again.  Slots >= n are ignored.  The outcome is the same for every lane; false = the wait expired.
-__device__ __forceinline__ bool take8(bool local, float* const (&p)[8], int n, float (&lo)[8], float (&hi)[8])
+// consumer side, whole wave: waits until the n (<= NMAX) word pairs at p[] all hold data, returns them and leaves the words
+// EMPTY again (n >= 1).  Slots >= n are ignored.  All requests of a round are in flight together.  The outcome is the same for
+// every lane; false = the wait expired.
+template <bool local, int NMAX>
+__device__ __forceinline__ bool take(float* const (&p)[NMAX], int n, float (&lo)[NMAX], float (&hi)[NMAX])
 {
-    uint64_t o[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = i < n ? EMPTY2 : 0;
+    uint64_t o[NMAX];
     int spins = 0;
     for (;;) {
+        asm volatile("" ::: "memory");                     // the words change under us: load them again every round
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            if (i < n && o[i] == EMPTY2) o[i] = local ? swap_l2(p[i]) : ld_dev64(p[i]);
+        for (int i = 0; i < NMAX; ++i) o[i] = local ? ld_l2(p[i < n ? i : 0]) : ld_dev64(p[i < n ? i : 0]);   // straight-line: all in flight together
         bool ok = true;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ok = ok && o[i] != EMPTY2;
+        for (int i = 0; i < NMAX; ++i) ok = ok && o[i] != EMPTY2;
         if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
         if (++spins >= SPIN_MAX) return false;
         __builtin_amdgcn_s_sleep(1);
     }
-    if (!local) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            if (i < n) st_dev64(p[i], EMPTY2);
+    for (int i = 0; i < NMAX; ++i) {                       // slots >= n repeat slot 0: no branches
+        if (local) *(uint64_t*)p[i < n ? i : 0] = EMPTY2; else st_dev64(p[i < n ? i : 0], EMPTY2);
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { lo[i] = __uint_as_float((uint32_t)o[i]); hi[i] = __uint_as_float((uint32_t)(o[i] >> 32)); }
+    for (int i = 0; i < NMAX; ++i) { lo[i] = __uint_as_float((uint32_t)o[i]); hi[i] = __uint_as_float((uint32_t)(o[i] >> 32)); }
     return true;
+}
+// the two activations k, k + 1 of a row (k even) as raw words: both loads are valid for every element type
+__device__ __forceinline__ void ld_x2_raw(const void* x, int xtype, int64_t i, uint32_t& r0, uint32_t& r1)
+{
+    const char* b = (const char*)x + i * (xtype == X_F32 ? 4 : 2);
+    r0 = *(const uint32_t*)b;
+    r1 = *(const uint32_t*)(xtype == X_F32 ? b + 4 : b);
+}
+__device__ __forceinline__ void cvt_x2(int xtype, uint32_t r0, uint32_t r1, float& v0, float& v1)
+{
+    if (xtype == X_F32) { v0 = __uint_as_float(r0); v1 = __uint_as_float(r1); }
+    else if (xtype == X_F16) { v0 = f16_bits_to_f32((uint16_t)r0); v1 = f16_bits_to_f32((uint16_t)(r0 >> 16)); }
+    else { v0 = __uint_as_float(r0 << 16); v1 = __uint_as_float(r0 & 0xffff0000u); }
 }
 
 struct Group { int e, n; };
@@ -153,16 +165,17 @@ __device__ __forceinline__ Group find_item(const FArgs& a, int g, int* sidx, uns
     return Group{e, misc[1]};
 }
 
-template <int CBK, int MR>
+template <int CBK, int MR, int TWA, bool LOCAL>
 __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
 {
-    __shared__ __align__(16) uint16_t xs[MR][KTB * 16];   // this block's K slice of the transformed activations (fp16)
+    __shared__ __align__(16) uint16_t xs[MR][FW * TWMAX * 16];   // this block's K slice of the transformed activations (fp16)
     __shared__ float red[FW][MR][128];
     __shared__ int sidx[PF_MAX], rows[RF_MAX], comb[RF_MAX], misc[4];
+    __shared__ float wsh[RF_MAX][16];                     // route weights of this item's token rows (stage 2)
     __shared__ unsigned char isf[PF_MAX];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bid = blockIdx.x;
-    const bool isA = bid < a.nA, local = a.local != 0;
+    const bool isA = bid < a.nA;
     const Exl3Cfg& c = a.c;
     // ---- block id -> work.  Group q lives on XCD q % 8: bid = ((q / 8) * bpg + j) * 8 + q % 8, j = position in the group.
     int g = -1, t = 0, nb = 0, s = 0, K, N;
@@ -186,7 +199,8 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
     TRACE(1);
     if (grp.n > 0) {
         const int Kt = K / 16, Nt = N / 16;
-        const int kt0 = s * KTB, kt1 = min(Kt, kt0 + KTB), nkt = kt1 - kt0;
+        const int ktb = FW * (isA ? TWA : TWB);           // k-tiles per block
+        const int kt0 = s * ktb, kt1 = min(Kt, kt0 + ktb), nkt = kt1 - kt0;
         const int nblk = (nkt + 7) / 8;                   // 128-blocks of K in this slice
         const uint32_t* tr = (const uint32_t*)a.tab[(int64_t)(isA ? t : 2) * c.E + grp.e];
         const int src = tile_prev_lane(lane);
@@ -199,17 +213,16 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
             const bool finisher = t == 1 && s == a.S1 - 1;
             // ---- the slice of x and its sign vector first (the transform overlaps the weight stream), then the tiles
             const uint16_t* suh = (const uint16_t*)a.tab[(int64_t)(3 + t) * c.E + grp.e];
-            float xv0 = 0.f, xv1 = 0.f;
+            uint32_t xr0 = 0, xr1 = 0, sr = 0;
             const int unit0 = wave;                       // first (row, 128-block) unit of this wave
             if (unit0 < grp.n * nblk) {
                 const int r = unit0 / nblk, kb = unit0 % nblk, k = kt0 * 16 + kb * 128 + 2 * lane;
-                const int64_t srow = rows[r] / c.topk;
-                xv0 = exl3_ld_x(a.x, c.xtype, srow * a.ldx + k) * f16_bits_to_f32(suh[k]);
-                xv1 = exl3_ld_x(a.x, c.xtype, srow * a.ldx + k + 1) * f16_bits_to_f32(suh[k + 1]);
+                ld_x2_raw(a.x, c.xtype, (int64_t)(rows[r] / c.topk) * a.ldx + k, xr0, xr1);
+                sr = *(const uint32_t*)(suh + k);
             }
-            uint4 wr[TW];
+            uint4 wr[TWA];
 #pragma unroll
-            for (int i = 0; i < TW; ++i) {
+            for (int i = 0; i < TWA; ++i) {
                 const int kt = kt0 + wave + FW * i;
                 wr[i] = make_uint4(0u, 0u, 0u, 0u);
                 if (kt < kt1) wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
@@ -228,20 +241,21 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
             // ---- transform the slice of x into LDS: wave per (row, 128-block)
             for (int u = unit0; u < grp.n * nblk; u += FW) {
                 const int r = u / nblk, kb = u % nblk;
-                float v0 = xv0, v1 = xv1;
                 if (u != unit0) {
                     const int k = kt0 * 16 + kb * 128 + 2 * lane;
-                    const int64_t srow = rows[r] / c.topk;
-                    v0 = exl3_ld_x(a.x, c.xtype, srow * a.ldx + k) * f16_bits_to_f32(suh[k]);
-                    v1 = exl3_ld_x(a.x, c.xtype, srow * a.ldx + k + 1) * f16_bits_to_f32(suh[k + 1]);
+                    ld_x2_raw(a.x, c.xtype, (int64_t)(rows[r] / c.topk) * a.ldx + k, xr0, xr1);
+                    sr = *(const uint32_t*)(suh + k);
                 }
+                float v0, v1;
+                cvt_x2(c.xtype, xr0, xr1, v0, v1);
+                v0 *= f16_bits_to_f32((uint16_t)sr); v1 *= f16_bits_to_f32((uint16_t)(sr >> 16));
                 fwht128(v0, v1, lane);
                 *(uint32_t*)&xs[r][kb * 128 + 2 * lane] = (uint32_t)f32_to_f16_bits(v0) | ((uint32_t)f32_to_f16_bits(v1) << 16);
             }
             __syncthreads();
             TRACE(3);
 #pragma unroll
-            for (int i = 0; i < TW; ++i) {
+            for (int i = 0; i < TWA; ++i) {
                 const int kt = kt0 + wave + FW * i;
                 if (kt < kt1) {
                     h2 wd[4][4];
@@ -265,28 +279,29 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
                     float v0 = red[0][r][col], v1 = red[0][r][col + 1];
 #pragma unroll
                     for (int w = 1; w < FW; ++w) { v0 += red[w][r][col]; v1 += red[w][r][col + 1]; }
-                    put2(local, &part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
+                    put2<LOCAL>(&part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
                 }
                 TRACE(6);
             } else {
                 // ---- finisher: gate and up sums in slice order, Hadamard, svh, activation, down input transform -> xh2
                 bool good = true;
                 for (int r = wave; r < grp.n; r += FW) {
-                    float gl[8], gh[8], ul[8], uh[8];
-                    float* pg[8]; float* pu[8];
+                    // gate slices 0 .. S1-1 and up slices 0 .. S1-2 (this block holds the last up slice itself), one round of requests
+                    float pl[2 * SMAX], ph[2 * SMAX];
+                    float* pp[2 * SMAX];
 #pragma unroll
-                    for (int ss = 0; ss < 8; ++ss) {
-                        const int s2 = ss < a.S1 ? ss : 0;
-                        pg[ss] = a.part1 + ((int64_t)(s2 * 2 + 0) * a.P + rows[r]) * c.I + ncol;
-                        pu[ss] = a.part1 + ((int64_t)(s2 * 2 + 1) * a.P + rows[r]) * c.I + ncol;
+                    for (int ss = 0; ss < 2 * SMAX; ++ss) {
+                        const int tt = ss < a.S1 ? 0 : 1, s2 = ss < a.S1 ? ss : (ss - a.S1 < a.S1 - 1 ? ss - a.S1 : 0);
+                        pp[ss] = a.part1 + ((int64_t)(s2 * 2 + tt) * a.P + rows[r]) * c.I + ncol;
                     }
-                    good = take8(local, pg, a.S1, gl, gh) && good;
-                    if (a.S1 > 1) good = take8(local, pu, a.S1 - 1, ul, uh) && good;
+                    good = take<LOCAL, 2 * SMAX>(pp, 2 * a.S1 - 1, pl, ph) && good;
+                    TRACE(4);
                     float g0 = 0.f, g1 = 0.f, u0 = 0.f, u1 = 0.f;
 #pragma unroll
-                    for (int ss = 0; ss < 8; ++ss) if (ss < a.S1) { g0 += gl[ss]; g1 += gh[ss]; }
-#pragma unroll
-                    for (int ss = 0; ss < 8; ++ss) if (ss < a.S1 - 1) { u0 += ul[ss]; u1 += uh[ss]; }
+                    for (int ss = 0; ss < 2 * SMAX; ++ss) {
+                        if (ss < a.S1) { g0 += pl[ss]; g1 += ph[ss]; }
+                        else if (ss < 2 * a.S1 - 1) { u0 += pl[ss]; u1 += ph[ss]; }
+                    }
                     float o0 = red[0][r][2 * lane], o1 = red[0][r][2 * lane + 1];      // this block's own slice of up, last in order
 #pragma unroll
                     for (int w = 1; w < FW; ++w) { o0 += red[w][r][2 * lane]; o1 += red[w][r][2 * lane + 1]; }
@@ -306,9 +321,9 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
             }
         } else {
             // ---- issue the tile loads, decode and fetch the finishing scales (independent of stage 1), then take xh2
-            uint4 wr[TW];
+            uint4 wr[TWB];
 #pragma unroll
-            for (int i = 0; i < TW; ++i) {
+            for (int i = 0; i < TWB; ++i) {
                 const int kt = kt0 + wave + FW * i;
                 wr[i] = make_uint4(0u, 0u, 0u, 0u);
                 if (kt < kt1) wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
@@ -319,6 +334,8 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
             const float svd0 = f16_bits_to_f32(svd[ncol]), svd1 = f16_bits_to_f32(svd[ncol + 1]);
             // rows of this item whose weighted sum this block does: those whose other experts all belong to earlier items
             if (finisher) {
+                for (int u = tid; u < grp.n * c.topk; u += 64 * FW)        // their route weights, fetched long before they are needed
+                    wsh[u / c.topk][u % c.topk] = exl3_ld_w(a.w, c.wtype, (rows[u / c.topk] / c.topk) * c.topk + u % c.topk);
                 if (a.R == 1) { if (tid == 0) comb[0] = g == a.P - 1; }
                 else {
                     if (tid < grp.n) comb[tid] = 1;
@@ -332,9 +349,13 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
                     }
                 }
             }
-            h2 wd[TW][4][4];
+            h2 wd[TWB][4][4];
 #pragma unroll
-            for (int i = 0; i < TW; ++i) decode_tile32<CBK>(wr[i], __shfl(wr[i].w, src, 64), wd[i]);
+            for (int i = 0; i < TWB; ++i) {
+                decode_tile32<CBK>(wr[i], __shfl(wr[i].w, src, 64), wd[i]);
+#pragma unroll
+                for (int q = 0; q < 16; ++q) asm volatile("" : "+v"(wd[i][q >> 2][q & 3]));   // decoded now, not after the wait
+            }
             asm volatile("" :: "v"(svd0), "v"(svd1));
             TRACE(3);
             __builtin_amdgcn_s_setprio(3);
@@ -364,7 +385,7 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
             TRACE(4);
             if (misc[2]) {
 #pragma unroll
-                for (int i = 0; i < TW; ++i) {
+                for (int i = 0; i < TWB; ++i) {
                     const int kt = kt0 + wave + FW * i;
                     if (kt < kt1) {
 #pragma unroll
@@ -385,7 +406,7 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
                         float v0 = red[0][r][col], v1 = red[0][r][col + 1];
 #pragma unroll
                         for (int w = 1; w < FW; ++w) { v0 += red[w][r][col]; v1 += red[w][r][col + 1]; }
-                        put2(local, &part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
+                        put2<LOCAL>(&part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
                     }
                     TRACE(6);
                 } else {
@@ -398,7 +419,7 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
                             float* pp[8];
 #pragma unroll
                             for (int ss = 0; ss < 8; ++ss) pp[ss] = a.part2 + ((int64_t)(ss < a.S2 - 1 ? ss : 0) * a.P + rows[r]) * c.H + ncol;
-                            ok = take8(local, pp, a.S2 - 1, pl, ph) && ok;
+                            ok = take<LOCAL, 8>(pp, a.S2 - 1, pl, ph) && ok;
 #pragma unroll
                             for (int ss = 0; ss < 8; ++ss) if (ss < a.S2 - 1) { v0 += pl[ss]; v1 += ph[ss]; }
                         }
@@ -407,32 +428,30 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
                         for (int w = 1; w < FW; ++w) { o0 += red[w][r][2 * lane]; o1 += red[w][r][2 * lane + 1]; }
                         v0 += o0; v1 += o1;
                         fwht128(v0, v1, lane);
-                        if (ok) put2(local, a.yd + (int64_t)rows[r] * c.H + ncol, v0 * svd0, v1 * svd1);
+                        if (ok) put2<LOCAL>(a.yd + (int64_t)rows[r] * c.H + ncol, v0 * svd0, v1 * svd1);
                     }
                     TRACE(6);
-                    // ---- rows this block sums: every expert's output of the row, in slot order, weighted
+                    // ---- token rows this block sums: every expert's output of the row, in slot order, weighted
                     for (int i = wave; i < grp.n; i += FW) {
                         if (!comb[i]) continue;
-                        const int r = rows[i] / c.topk;
+                        const int tr = rows[i] / c.topk;
+                        const float b0 = a.add ? a.add[(int64_t)tr * c.H + ncol] : 0.f, b1 = a.add ? a.add[(int64_t)tr * c.H + ncol + 1] : 0.f;
+                        float yl[16], yh[16];
+                        float* py[16];
+#pragma unroll
+                        for (int k = 0; k < 16; ++k) py[k] = a.yd + (int64_t)(tr * c.topk + (k < c.topk ? k : 0)) * c.H + ncol;
+                        ok = take<LOCAL, 16>(py, c.topk, yl, yh) && ok;
+                        TRACE(2);
                         float a0 = 0.f, a1 = 0.f;
-                        for (int k0 = 0; k0 < c.topk; k0 += 8) {                // 8 experts' outputs requested together
-                            float yl[8], yh[8];
-                            float* py[8];
-                            const int nk = min(8, c.topk - k0);
 #pragma unroll
-                            for (int k = 0; k < 8; ++k) py[k] = a.yd + (int64_t)(r * c.topk + k0 + (k < nk ? k : 0)) * c.H + ncol;
-                            ok = take8(local, py, nk, yl, yh) && ok;
-#pragma unroll
-                            for (int k = 0; k < 8; ++k)
-                                if (k < nk) {
-                                    const float wk = exl3_ld_w(a.w, c.wtype, r * c.topk + k0 + k);
-                                    a0 += wk * yl[k]; a1 += wk * yh[k];
-                                }
-                        }
-                        const float b0 = a.add ? a.add[(int64_t)r * c.H + ncol] : 0.f, b1 = a.add ? a.add[(int64_t)r * c.H + ncol + 1] : 0.f;
+                        for (int k = 0; k < 16; ++k)
+                            if (k < c.topk) {
+                                const float wk = wsh[i][k];
+                                a0 += wk * yl[k]; a1 += wk * yh[k];
+                            }
                         if (ok) {
-                            a.out[(int64_t)r * c.H + ncol] = b0 + a0;
-                            a.out[(int64_t)r * c.H + ncol + 1] = b1 + a1;
+                            a.out[(int64_t)tr * c.H + ncol] = b0 + a0;
+                            a.out[(int64_t)tr * c.H + ncol + 1] = b1 + a1;
                         }
                     }
                     if (!ok && lane == 0) atomicExch(a.err, 1);
@@ -455,14 +474,16 @@ __global__ void xcd_probe_kernel(int* out)
     if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((31 << 11) | 20) & 0xf;
 }
 
-struct FPlan { int P, Gmax, S1, S2, NB1, NB2, nA, nB, bpgA, bpgB; size_t part1, xh2, part2, yd, total; };
+struct FPlan { int P, Gmax, twa, S1, S2, NB1, NB2, nA, nB, bpgA, bpgB; size_t part1, xh2, part2, yd, total; };
 FPlan fplan(const Exl3Cfg& c, int R)
 {
     FPlan p;
     p.P = R * c.topk;
     p.Gmax = p.P < c.E ? p.P : c.E;
-    p.S1 = (c.H / 16 + KTB - 1) / KTB;
-    p.S2 = (c.I / 16 + KTB - 1) / KTB;
+    // finer stage-1 blocks balance the CUs better while the grid is small (and K allows 8 slices)
+    p.twa = c.H / 16 <= SMAX * FW * 4 && (int64_t)p.Gmax * (c.I / 128) * 2 * (c.H / 16 / (FW * 4)) <= 1024 ? 4 : 8;
+    p.S1 = (c.H / 16 + FW * p.twa - 1) / (FW * p.twa);
+    p.S2 = (c.I / 16 + FW * TWB - 1) / (FW * TWB);
     p.NB1 = c.I / 128; p.NB2 = c.H / 128;
     p.bpgA = 2 * p.S1; p.bpgB = p.Gmax * p.S2;
     const int QA = (p.Gmax * p.NB1 + NXCD - 1) / NXCD * NXCD, QB = (p.NB2 + NXCD - 1) / NXCD * NXCD;   // groups, padded to the XCD count
@@ -478,15 +499,21 @@ FPlan fplan(const Exl3Cfg& c, int R)
     return p;
 }
 
-template <int CBK>
-void launch(const FArgs& a, int maxrows, hipStream_t st)
+template <int CBK, int TWA, bool LOCAL>
+void launch3(const FArgs& a, int maxrows, hipStream_t st)
 {
     const dim3 grid(a.nA + a.nB), blk(64 * FW);
-    if (maxrows <= 1) fused_kernel<CBK, 1><<<grid, blk, 0, st>>>(a);
-    else if (maxrows <= 2) fused_kernel<CBK, 2><<<grid, blk, 0, st>>>(a);
-    else if (maxrows <= 4) fused_kernel<CBK, 4><<<grid, blk, 0, st>>>(a);
-    else if (maxrows <= 8) fused_kernel<CBK, 8><<<grid, blk, 0, st>>>(a);
-    else fused_kernel<CBK, 16><<<grid, blk, 0, st>>>(a);
+    if (maxrows <= 1) fused_kernel<CBK, 1, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
+    else if (maxrows <= 2) fused_kernel<CBK, 2, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
+    else if (maxrows <= 4) fused_kernel<CBK, 4, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
+    else if (maxrows <= 8) fused_kernel<CBK, 8, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
+    else fused_kernel<CBK, 16, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
+}
+template <int CBK>
+void launch(const FArgs& a, int twa, int maxrows, hipStream_t st)
+{
+    if (a.local) { if (twa == 4) launch3<CBK, 4, true>(a, maxrows, st); else launch3<CBK, 8, true>(a, maxrows, st); }
+    else { if (twa == 4) launch3<CBK, 4, false>(a, maxrows, st); else launch3<CBK, 8, false>(a, maxrows, st); }
 }
 
 int g_xcd_local = -1;                 // -1 unknown, 0 placement check failed, 1 workgroup b runs on XCD b % 8
@@ -495,7 +522,7 @@ int g_xcd_local = -1;                 // -1 unknown, 0 placement check failed, 1
 
 bool exl3_fused_ok(const Exl3Cfg& c, int R)
 {
-    return R >= 1 && R <= RF_MAX && R * c.topk <= PF_MAX && c.H <= SMAX * KTB * 16 && c.I <= SMAX * KTB * 16;
+    return R >= 1 && R <= RF_MAX && c.topk <= 16 && R * c.topk <= PF_MAX && c.H <= SMAX * FW * TWMAX * 16 && c.I <= SMAX * FW * TWB * 16;
 }
 size_t exl3_fused_ws_bytes(const Exl3Cfg& c, int R) { return fplan(c, R).total; }
 
@@ -543,8 +570,8 @@ int exl3_fused_launch(const Exl3Cfg& c, const void* x, int64_t ldx, int R, const
         const int rc = exl3_fused_ws_prepare(ws, p.total, st);
         if (rc) return rc;
     }
-    if (c.cbk == CB_MCG) launch<CB_MCG>(a, R, st);
-    else launch<CB_MUL1>(a, R, st);
+    if (c.cbk == CB_MCG) launch<CB_MCG>(a, p.twa, R, st);
+    else launch<CB_MUL1>(a, p.twa, R, st);
     return launch_status();
 }
 
