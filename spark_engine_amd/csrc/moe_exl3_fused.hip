@@ -193,6 +193,13 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
     }
     if (isA) __builtin_amdgcn_s_setprio(2);               // stage 1 is the critical path: its waves issue first
     TRACE(0);
+    // Warm this XCD's L2 with the expert table while the routing indices are on their way: the table lookup that follows
+    // them is a dependent access and would otherwise go to memory.  The blocks of an XCD cover the table once.
+    uint64_t warm = 0;
+    {
+        const int64_t i = (int64_t)(bid / NXCD) * (64 * FW) + tid;
+        if (i < (int64_t)9 * c.E) warm = a.tab[i];
+    }
     if (tid == 0) misc[2] = 1;
     Group grp{0, 0};
     if (g >= 0) grp = find_item(a, g, sidx, isf, rows, misc);
@@ -213,19 +220,21 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
             const bool finisher = t == 1 && s == a.S1 - 1;
             // ---- the slice of x and its sign vector first (the transform overlaps the weight stream), then the tiles
             const uint16_t* suh = (const uint16_t*)a.tab[(int64_t)(3 + t) * c.E + grp.e];
-            uint32_t xr0 = 0, xr1 = 0, sr = 0;
+            uint32_t xr0, xr1, sr;
             const int unit0 = wave;                       // first (row, 128-block) unit of this wave
-            if (unit0 < grp.n * nblk) {
-                const int r = unit0 / nblk, kb = unit0 % nblk, k = kt0 * 16 + kb * 128 + 2 * lane;
+            {
+                // no branch around these loads (a wave without a unit fetches unit 0 again): their wait must not land
+                // ahead of the tile loads
+                const int uu = unit0 < grp.n * nblk ? unit0 : 0;
+                const int r = uu / nblk, kb = uu % nblk, k = kt0 * 16 + kb * 128 + 2 * lane;
                 ld_x2_raw(a.x, c.xtype, (int64_t)(rows[r] / c.topk) * a.ldx + k, xr0, xr1);
                 sr = *(const uint32_t*)(suh + k);
             }
             uint4 wr[TWA];
 #pragma unroll
             for (int i = 0; i < TWA; ++i) {
-                const int kt = kt0 + wave + FW * i;
-                wr[i] = make_uint4(0u, 0u, 0u, 0u);
-                if (kt < kt1) wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
+                const int kt = min(kt0 + wave + FW * i, kt1 - 1);          // past the slice: a valid tile again, unused (no branch around a load)
+                wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
             }
             TRACE(2);
             // ---- scales of the finishing step (the finisher only)
@@ -324,9 +333,8 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
             uint4 wr[TWB];
 #pragma unroll
             for (int i = 0; i < TWB; ++i) {
-                const int kt = kt0 + wave + FW * i;
-                wr[i] = make_uint4(0u, 0u, 0u, 0u);
-                if (kt < kt1) wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
+                const int kt = min(kt0 + wave + FW * i, kt1 - 1);          // past the slice: a valid tile again, unused (no branch around a load)
+                wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
             }
             TRACE(2);
             const bool finisher = s == a.S2 - 1;
@@ -358,7 +366,6 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
             }
             asm volatile("" :: "v"(svd0), "v"(svd1));
             TRACE(3);
-            __builtin_amdgcn_s_setprio(3);
             uint32_t* xc = a.xh2 + ((int64_t)nb * a.P) * (c.I / 2) + kt0 * 8;         // this column block's copy, this K slice
             // cheap wait first: one word per 128-block of the slice (the finishers' last lanes), then every word
             if (wave == 0) {
@@ -366,10 +373,11 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
                 for (;;) {
                     const uint32_t v = lane < nblk ? ld_dev32(xc + (int64_t)rows[0] * (c.I / 2) + lane * 64 + 63) : 0u;
                     if (__builtin_amdgcn_ballot_w64(v == EMPTY) == 0 || ++spins >= SPIN_MAX) break;
-                    __builtin_amdgcn_s_sleep(2);
+                    __builtin_amdgcn_s_sleep(4);
                 }
             }
             __syncthreads();
+            __builtin_amdgcn_s_setprio(3);                // from here on this block is the critical path
             bool good = true;
             for (int u = tid; u < grp.n * (nkt * 8); u += 64 * FW) {                  // 2 fp16 per thread-step
                 const int r = u / (nkt * 8), q = u % (nkt * 8);
@@ -459,6 +467,7 @@ __global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
             } else if (tid == 0) atomicExch(a.err, 1);
         }
     }
+    asm volatile("" :: "v"(warm));                         // the warming load is complete before the wave ends
     TRACE(7);
 }
 
