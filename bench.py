@@ -137,8 +137,7 @@ class Mxfp4Layer:
         self.idx = torch.empty(inst, R, self.TOPK, dtype=torch.int64, device=dev)
         self.rw = torch.empty(inst, R, self.TOPK, dtype=torch.float32, device=dev)
         self.y = torch.empty(inst, R, H, dtype=torch.float32, device=dev)
-        self.ws = torch.empty(ops.mxfp4_moe_ws(R, self.ex, self.TOPK), dtype=torch.uint8, device=dev)
-        self.scratch = (torch.empty(R, H, dtype=torch.uint8, device=dev), torch.empty(R, H // 32, dtype=torch.uint8, device=dev))
+        self.ws = ops.mxfp4_moe_ws_alloc(R, self.ex, self.TOPK)
         self.name = f"C3 deepseek-style MXFP4 MoE layer (H {H}, I {I}, {self.E} experts top-{self.TOPK} + {self.NS} shared), batch {R}"
 
     def step(self, i):
@@ -146,7 +145,13 @@ class Mxfp4Layer:
         st = ops._st()
         k = i % self.inst
         ops._ck(L.ds41_route(ops._p(self.logits[k]), ops._p(self.bias), ops._p(self.idx[k]), ops._p(self.rw[k]), self.R, self.E, self.TOPK, 1.5, st), "route")
-        ops.mxfp4_moe(self.x, self.idx[k], self.rw[k], self.ex, y=self.y[k], ws=self.ws, scratch=self.scratch)
+        ops.mxfp4_moe_x(self.x, self.idx[k], self.rw[k], self.ex, y=self.y[k], ws=self.ws, ws_clean=True)
+
+    DOMINANT = "spk::mx::mx_fused_kernel (the single-launch routed-experts kernel of spark_mxfp4_moe_x)"
+
+    def dominant(self, i):
+        k = i % self.inst
+        self.ops.mxfp4_moe_x(self.x, self.idx[k], self.rw[k], self.ex, y=self.y[k], ws=self.ws, ws_clean=True)
 
     def bytes_per_step(self):
         idx = self.idx.cpu().numpy()

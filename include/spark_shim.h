@@ -113,6 +113,14 @@ SPARK_API int spark_mxfp4_moe_q(const void* xq, const void* xs, int R, const int
 SPARK_API int spark_mxfp4_moe(const void* x, void* xq, void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1,
                               const void* w3, const void* s3, const void* w2, const void* s2, int layout, int H, int I, int topk, int E,
                               int n_shared, const float* add, float* y, void* ws, hipStream_t st);
+/* Decode entry (R <= 8 token rows, topk + n_shared <= 16): the whole layer as ONE launch.  x is bf16 [R, H] when xs is NULL (act_quant
+ * runs inside the kernel) or E4M3 [R, H] with its E8M0 scales xs.  flags bit 0: ws was prepared by spark_mxfp4_moe_ws_init (call it
+ * once after allocating ws, outside stream capture) and only used by this entry point since; without it one more launch prepares ws
+ * first.  flags bit 1: use the several-kernel path (xs required).  Same values, bit for bit, as the several-kernel path. */
+SPARK_API int spark_mxfp4_moe_ws_init(void* ws, size_t bytes, hipStream_t st);
+SPARK_API int spark_mxfp4_moe_x(const void* x, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1,
+                                const void* w3, const void* s3, const void* w2, const void* s2, int layout, int H, int I, int topk, int E,
+                                int n_shared, const float* add, float* y, void* ws, int flags, hipStream_t st);
 /* The reference's DeepSeek entry points (H = 5120 as compiled there, weights in the moe_pack_mx layout with raw scale bytes).
  * Replace engine-rs/shim/ds41_mx.cu:1426-1523.  ds41_moe_mx_ws_ptrs hands out the per-pair down output [P, H] fp32 and pairmap [P]
  * inside ws, valid after ds41_moe_mx_ex(skip_combine = 1). */

@@ -19,91 +19,19 @@
 // Weight storage ("T16" records, written once by spark_mxfp4_prepack): per 16 rows and 512-wide K group one record of
 // 4352 bytes = 4 steps x (64 lanes x 16 bytes of codes) + 64 lanes x 4 scale bytes (byte s = step s).  A wave streams a
 // record with four 16-byte loads and one 4-byte load per lane, all contiguous.
-#include "common.hpp"
+#include "moe_mxfp4.hpp"
 
 using namespace spk;
+using namespace spk::mx;
 
 namespace {
 
 struct Item { int e, off, n, pad; };
 
-constexpr int REC = 4352;              // bytes per T16 record
 constexpr int EMAXG = 2048;            // experts the grouping kernel can hold
 constexpr int UP_WAVES = 8, DN_WAVES = 4;
 
-enum Layout { L_T16 = 0, L_NATURAL = 1, L_PACK8 = 2, L_MX8 = 3 };
 
-struct WMat {                          // one stacked weight matrix [E, rows, K]
-    const uint8_t* w;
-    const uint8_t* s;
-    int rows, K;                       // per expert
-};
-
-// ---- A operand: the 4 steps of K group kg of the 16 rows starting at row0 (row0 % 16 == 0) of expert e
-template <int LAYOUT>
-__device__ __forceinline__ void load_group(const WMat& m, int e, int row0, int kg, int lane, v4i (&c)[4], uint32_t& sc4)
-{
-    const int r = lane & 15, g = lane >> 4, steps = m.K >> 7, nkg = (steps + 3) >> 2;
-    if constexpr (LAYOUT == L_T16) {
-        const int64_t tile = ((int64_t)e * m.rows + row0) >> 4;
-        const uint8_t* rec = m.w + (tile * nkg + kg) * REC;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) { const uint4 v = ld_stream16(rec + s * 1024 + lane * 16); c[s] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}; }
-        sc4 = __builtin_nontemporal_load((const uint32_t*)(rec + 4096 + lane * 4));
-    } else {
-        sc4 = 0x7f7f7f7fu;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const int step = kg * 4 + s;
-            c[s] = v4i{0, 0, 0, 0};
-            if (step >= steps) continue;
-            const int64_t row = (int64_t)e * m.rows + row0 + r;
-            uint32_t sb;
-            if constexpr (LAYOUT == L_NATURAL) {
-                const uint4 v = ld_stream16(m.w + row * (m.K >> 1) + step * 64 + g * 16);
-                c[s] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-                sb = m.s[row * (m.K >> 5) + step * 4 + g];
-            } else if constexpr (LAYOUT == L_PACK8) {      // [rows/8][K/128][8][4][16], scales [rows/8][K/128][8][4]
-                const int64_t t8 = row >> 3;
-                const uint4 v = ld_stream16(m.w + (t8 * steps + step) * 512 + (row & 7) * 64 + g * 16);
-                c[s] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-                sb = m.s[(t8 * steps + step) * 32 + (row & 7) * 4 + g];
-            } else {                                        // L_MX8: [rows/8][K/128][8][4 q][4 b][4]
-                const int64_t t8 = row >> 3;
-                const uint32_t* p = (const uint32_t*)(m.w + (t8 * steps + step) * 512 + (row & 7) * 64 + g * 4);
-                c[s] = v4i{(int)p[0], (int)p[4], (int)p[8], (int)p[12]};
-                sb = m.s[(t8 * steps + step) * 32 + (row & 7) * 4 + g];
-            }
-            sc4 = (sc4 & ~(0xffu << (8 * s))) | (sb << (8 * s));
-        }
-    }
-}
-
-// ---- B operand of one step: E4M3 bytes of row `q` (row stride K) + its UE8M0 scales (row stride K/32)
-__device__ __forceinline__ void load_b(const uint8_t* __restrict__ q, const uint8_t* __restrict__ qs, int step, int lane, v8i& b, uint32_t& sb)
-{
-    const int g = lane >> 4;
-    const uint4 lo = *(const uint4*)(q + step * 128 + 16 * g);
-    const uint4 hi = *(const uint4*)(q + step * 128 + 64 + 16 * g);
-    b = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-    sb = qs[step * 4 + g];
-}
-
-template <int OPSEL>
-__device__ __forceinline__ v4f mfma_step(const v4i& a, const v8i& b, v4f acc, uint32_t sa, uint32_t sb)
-{
-    const v8i a8 = v8i{a.x, a.y, a.z, a.w, 0, 0, 0, 0};
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b, acc, 4 /*A: E2M1*/, 0 /*B: E4M3*/, OPSEL, (int)sa, 0, (int)sb);
-}
-__device__ __forceinline__ v4f mfma_group_step(int s, const v4i& a, const v8i& b, v4f acc, uint32_t sa4, uint32_t sb)
-{
-    switch (s) {
-        case 0: return mfma_step<0>(a, b, acc, sa4, sb);
-        case 1: return mfma_step<1>(a, b, acc, sa4, sb);
-        case 2: return mfma_step<2>(a, b, acc, sa4, sb);
-        default: return mfma_step<3>(a, b, acc, sa4, sb);
-    }
-}
 
 // ---------------------------------------------------------------- grouping of the (row, expert) pairs by expert
 // Pairs per row: topk routed (idx, rw) followed by n_shared shared experts (ids E .. E + n_shared - 1, weight 1).
@@ -414,11 +342,25 @@ SPARK_API int spark_mxfp4_prepack(const void* w, const void* s, void* packed, lo
     prepack_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((const uint8_t*)w, (const uint8_t*)s, (uint8_t*)packed, tiles, K);
     return launch_status();
 }
+// the single-launch path's workspace follows the several-kernel path's (they never share bytes)
 SPARK_API size_t spark_mxfp4_moe_ws_bytes(int R, int H, int I, int topk, int E, int n_shared)
 {
     if (!shapes_ok(R, H, I, topk, E, n_shared)) return 0;
-    return ws_layout(R, H, I, topk + n_shared, E + n_shared).total;
+    return ws_layout(R, H, I, topk + n_shared, E + n_shared).total + (mx_fused_ok(R, H, I, topk, E, n_shared) ? mx_fused_ws_bytes(R, H, I, topk, E, n_shared) : 0);
 }
+// prepares a workspace once after allocation (not under stream capture: it also checks workgroup placement, which synchronises);
+// calls of spark_mxfp4_moe_x with flags bit 0 then skip their own preparing launch
+SPARK_API int spark_mxfp4_moe_ws_init(void* ws, size_t bytes, hipStream_t st)
+{
+    mx_xcd_probe();
+    return mx_fused_ws_prepare(ws, bytes, st);
+}
+namespace {
+inline void* fused_ws(void* ws, int R, int H, int I, int topk, int E, int n_shared)
+{
+    return (char*)ws + ws_layout(R, H, I, topk + n_shared, E + n_shared).total;
+}
+}  // namespace
 // xq [R, H] E4M3 + xs [R, H/32] UE8M0 (act_quant of x); idx int64 / rw f32 [R, topk]; stacked weights of E + n_shared
 // experts: layout 0 = T16 records (s* unused), 1 = natural [E, rows, K/2] + [E, rows, K/32]; the n_shared experts after
 // the E routed ones run on every row with weight 1; add [R, H] f32 or null; y [R, H] f32.
@@ -426,25 +368,46 @@ SPARK_API int spark_mxfp4_moe_q(const void* xq, const void* xs, int R, const int
                                 const void* s3, const void* w2, const void* s2, int layout, int H, int I, int topk, int E, int n_shared, const float* add,
                                 float* y, void* ws, hipStream_t st)
 {
-    if (!shapes_ok(R, H, I, topk, E, n_shared)) return 1;
+    if (!shapes_ok(R, H, I, topk, E, n_shared) || (layout != L_T16 && layout != L_NATURAL)) return 1;
+    if (mx_fused_ok(R, H, I, topk, E, n_shared))
+        return mx_fused_launch(xq, xs, R, idx, rw, w1, s1, w3, s3, w2, s2, layout, H, I, topk, E, n_shared, add, y, fused_ws(ws, R, H, I, topk, E, n_shared), 0, st);
     if (layout == L_T16)
         return moe_launch<L_T16>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, nullptr, (const uint8_t*)w3, nullptr, (const uint8_t*)w2,
                                  nullptr, H, I, topk, E, n_shared, add, y, ws, 0, st);
-    if (layout == L_NATURAL)
-        return moe_launch<L_NATURAL>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3,
-                                     (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, H, I, topk, E, n_shared, add, y, ws, 0, st);
-    return 1;
+    return moe_launch<L_NATURAL>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3,
+                                 (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, H, I, topk, E, n_shared, add, y, ws, 0, st);
 }
 extern "C" int ds41_act_quant_fp8(const void* x, void* q, void* s, long long numel, hipStream_t st);
-// x bf16 [R, H]: act_quant per 32 first (scratch xq, xs from the caller: R*H and R*H/32 bytes), then spark_mxfp4_moe_q
+// x bf16 [R, H]: act_quant per 32 first (scratch xq, xs from the caller: R*H and R*H/32 bytes, used beyond 8 rows), then the experts
 SPARK_API int spark_mxfp4_moe(const void* x, void* xq, void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3,
                               const void* s3, const void* w2, const void* s2, int layout, int H, int I, int topk, int E, int n_shared, const float* add, float* y,
                               void* ws, hipStream_t st)
 {
-    if (!shapes_ok(R, H, I, topk, E, n_shared)) return 1;
+    if (!shapes_ok(R, H, I, topk, E, n_shared) || (layout != L_T16 && layout != L_NATURAL)) return 1;
+    if (mx_fused_ok(R, H, I, topk, E, n_shared))
+        return mx_fused_launch(x, nullptr, R, idx, rw, w1, s1, w3, s3, w2, s2, layout, H, I, topk, E, n_shared, add, y, fused_ws(ws, R, H, I, topk, E, n_shared), 0, st);
     const int rc = ds41_act_quant_fp8(x, xq, xs, (long long)R * H, st);
     if (rc) return rc;
     return spark_mxfp4_moe_q(xq, xs, R, idx, rw, w1, s1, w3, s3, w2, s2, layout, H, I, topk, E, n_shared, add, y, ws, st);
+}
+// The decode entry: x bf16 [R, H] with xs null (quantised inside the kernel) or E4M3 with scales xs; R <= 8, topk + n_shared <= 16.
+// flags bit 0: ws was prepared by spark_mxfp4_moe_ws_init and has only been used by this entry point since (one launch in all);
+// flags bit 1: use the several-kernel path (xs must be given).
+SPARK_API int spark_mxfp4_moe_x(const void* x, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3,
+                                const void* s3, const void* w2, const void* s2, int layout, int H, int I, int topk, int E, int n_shared, const float* add, float* y,
+                                void* ws, int flags, hipStream_t st)
+{
+    if (!shapes_ok(R, H, I, topk, E, n_shared) || (layout != L_T16 && layout != L_NATURAL)) return 1;
+    if (flags & 2) {
+        if (!xs) return 1;
+        if (layout == L_T16)
+            return moe_launch<L_T16>((const uint8_t*)x, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, nullptr, (const uint8_t*)w3, nullptr,
+                                     (const uint8_t*)w2, nullptr, H, I, topk, E, n_shared, add, y, ws, 0, st);
+        return moe_launch<L_NATURAL>((const uint8_t*)x, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3,
+                                     (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, H, I, topk, E, n_shared, add, y, ws, 0, st);
+    }
+    if (!mx_fused_ok(R, H, I, topk, E, n_shared)) return 1;
+    return mx_fused_launch(x, xs, R, idx, rw, w1, s1, w3, s3, w2, s2, layout, H, I, topk, E, n_shared, add, y, fused_ws(ws, R, H, I, topk, E, n_shared), flags & 1, st);
 }
 
 // ================================================================ C ABI: the reference's symbols (hidden size 5120)

@@ -1,0 +1,101 @@
+// Shared pieces of the MXFP4 expert kernels: weight layouts, the A / B operand loads and the block-scaled MFMA step.
+//
+// Operand layout of v_mfma_scale_f32_16x16x128_f8f6f4 measured on gfx950: A/B lane l = row/column l % 16, K group g = l / 16.
+// An E2M1 operand holds k = 32 g + e (nibble e of its 16 bytes); an E4M3 operand holds k = 16 g + e in registers 0-3 and
+// k = 64 + 16 g + e in registers 4-7; the scale byte of lane l applies to logical block g (k in [32 g, 32 g + 32)); D lane l =
+// column l % 16, rows 4 (l / 16) + {0..3}.
+#pragma once
+#include "common.hpp"
+
+namespace spk {
+namespace mx {
+
+constexpr int REC = 4352;              // bytes per T16 record
+
+enum Layout { L_T16 = 0, L_NATURAL = 1, L_PACK8 = 2, L_MX8 = 3 };
+
+struct WMat {                          // one stacked weight matrix [E, rows, K]
+    const uint8_t* w;
+    const uint8_t* s;
+    int rows, K;                       // per expert
+};
+
+// ---- A operand: the 4 steps of K group kg of the 16 rows starting at row0 (row0 % 16 == 0) of expert e
+template <int LAYOUT>
+__device__ __forceinline__ void load_group(const WMat& m, int e, int row0, int kg, int lane, v4i (&c)[4], uint32_t& sc4)
+{
+    const int r = lane & 15, g = lane >> 4, steps = m.K >> 7, nkg = (steps + 3) >> 2;
+    if constexpr (LAYOUT == L_T16) {
+        const int64_t tile = ((int64_t)e * m.rows + row0) >> 4;
+        const uint8_t* rec = m.w + (tile * nkg + kg) * REC;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { const uint4 v = ld_stream16(rec + s * 1024 + lane * 16); c[s] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w}; }
+        sc4 = __builtin_nontemporal_load((const uint32_t*)(rec + 4096 + lane * 4));
+    } else {
+        sc4 = 0x7f7f7f7fu;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int step = kg * 4 + s;
+            c[s] = v4i{0, 0, 0, 0};
+            if (step >= steps) continue;
+            const int64_t row = (int64_t)e * m.rows + row0 + r;
+            uint32_t sb;
+            if constexpr (LAYOUT == L_NATURAL) {
+                const uint4 v = ld_stream16(m.w + row * (m.K >> 1) + step * 64 + g * 16);
+                c[s] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                sb = m.s[row * (m.K >> 5) + step * 4 + g];
+            } else if constexpr (LAYOUT == L_PACK8) {      // [rows/8][K/128][8][4][16], scales [rows/8][K/128][8][4]
+                const int64_t t8 = row >> 3;
+                const uint4 v = ld_stream16(m.w + (t8 * steps + step) * 512 + (row & 7) * 64 + g * 16);
+                c[s] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                sb = m.s[(t8 * steps + step) * 32 + (row & 7) * 4 + g];
+            } else {                                        // L_MX8: [rows/8][K/128][8][4 q][4 b][4]
+                const int64_t t8 = row >> 3;
+                const uint32_t* p = (const uint32_t*)(m.w + (t8 * steps + step) * 512 + (row & 7) * 64 + g * 4);
+                c[s] = v4i{(int)p[0], (int)p[4], (int)p[8], (int)p[12]};
+                sb = m.s[(t8 * steps + step) * 32 + (row & 7) * 4 + g];
+            }
+            sc4 = (sc4 & ~(0xffu << (8 * s))) | (sb << (8 * s));
+        }
+    }
+}
+
+// ---- B operand of one step: E4M3 bytes of row `q` (row stride K) + its UE8M0 scales (row stride K/32)
+__device__ __forceinline__ void load_b(const uint8_t* __restrict__ q, const uint8_t* __restrict__ qs, int step, int lane, v8i& b, uint32_t& sb)
+{
+    const int g = lane >> 4;
+    const uint4 lo = *(const uint4*)(q + step * 128 + 16 * g);
+    const uint4 hi = *(const uint4*)(q + step * 128 + 64 + 16 * g);
+    b = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    sb = qs[step * 4 + g];
+}
+
+template <int OPSEL>
+__device__ __forceinline__ v4f mfma_step(const v4i& a, const v8i& b, v4f acc, uint32_t sa, uint32_t sb)
+{
+    const v8i a8 = v8i{a.x, a.y, a.z, a.w, 0, 0, 0, 0};
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b, acc, 4 /*A: E2M1*/, 0 /*B: E4M3*/, OPSEL, (int)sa, 0, (int)sb);
+}
+__device__ __forceinline__ v4f mfma_group_step(int s, const v4i& a, const v8i& b, v4f acc, uint32_t sa4, uint32_t sb)
+{
+    switch (s) {
+        case 0: return mfma_step<0>(a, b, acc, sa4, sb);
+        case 1: return mfma_step<1>(a, b, acc, sa4, sb);
+        case 2: return mfma_step<2>(a, b, acc, sa4, sb);
+        default: return mfma_step<3>(a, b, acc, sa4, sb);
+    }
+}
+
+// ---- the single-launch decode path (moe_mxfp4_fused.hip): R <= 8 token rows, topk + shared <= 16
+bool mx_fused_ok(int R, int H, int I, int topk, int E, int n_shared);
+size_t mx_fused_ws_bytes(int R, int H, int I, int topk, int E, int n_shared);
+int mx_xcd_probe();
+int mx_fused_ws_prepare(void* ws, size_t bytes, hipStream_t st);
+// x: bf16 [R, H] when xs is null (quantised inside), else E4M3 [R, H] with its scales xs.  clean: the exchanged words of ws are
+// idle (prepared once and only used by this path since); otherwise one more launch prepares them first.
+int mx_fused_launch(const void* x, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3, const void* s3,
+                    const void* w2, const void* s2, int layout, int H, int I, int topk, int E, int n_shared, const float* add, float* y, void* ws, int clean,
+                    hipStream_t st);
+
+}  // namespace mx
+}  // namespace spk

@@ -1,0 +1,517 @@
+// Routed MXFP4 experts (gate / up, SwiGLU, act_quant, down, weighted sum) in ONE launch for decode-sized calls:
+// R <= 8 token rows, topk + shared <= 16 experts per row.
+//
+// The several-kernel path (moe_mxfp4.hip) spends more time in launch gaps and tiny kernels (activation quantisation,
+// grouping, combine) than the batch-1 weight stream takes.  Here one grid holds both weight streams:
+//   U blocks: (item, 32 features of I).  8 waves split K as in up_kernel (same summation order, so the values are the
+//       same bits): each wave quantises its K groups of the token rows itself (act_quant per 32, into LDS), streams the 32
+//       gate and 32 up rows, block-scaled MFMA, LDS reduction in wave order, SwiGLU * route weight, act_quant of the 32
+//       features; the 32 code bytes + scale of every item row go to every stage-2 column block's own copy of h.
+//   D blocks: (64 output columns | item).  Stream their down-projection rows into registers first (raw MXFP4 is the MFMA
+//       operand, nothing to decode), then take the item's h, MFMA as in down_kernel (same order), hand the per-pair
+//       outputs over inside the XCD; for every token row the block of the row's last item in launch order adds
+//       them up: (add + shared experts) + (routed experts in slot order), the reference's order.
+//
+// Exchange without counters: every exchanged 32-bit word of the workspace is EMPTY (all ones) between uses; a producer
+// stores its value (an all-ones value is altered to another NaN pattern), the single consumer of the word polls until it
+// is not EMPTY and stores EMPTY back.  h crosses XCDs (device-coherent stores and loads), the per-pair outputs stay in
+// one XCD's L2 (workgroup b runs on XCD b % 8; all D blocks of a column block share an XCD).  A block only waits for blocks
+// with lower ids; waits are bounded and an expiry raises an error flag while every block still runs to its end.
+//
+// Semantics: reference engine-rs/shim/ds41_moe.cu:1-24, ds41_mx.cu:129-317, engine-rs/src/ds41/kern.rs:1116-1133.
+#include "moe_mxfp4.hpp"
+
+namespace spk {
+namespace mx {
+namespace {
+
+constexpr int NW = 8, NT = 64 * NW;
+constexpr int RMAX = 8, TTMAX = 16, PMAXF = RMAX * TTMAX;
+constexpr int DC = 64;                 // output columns of a stage-2 block
+constexpr int NXCD = 8, HEAD = 256, SPIN_MAX = 200000;
+constexpr uint32_t EMPTY = 0xffffffffu;
+constexpr uint64_t EMPTY2 = ~0ull;
+constexpr int RED_BYTES = NW * 4 * 4 * 64 * 4;
+
+struct MArgs {
+    const void* x;                     // bf16 [R, H] (QUANT) or E4M3 [R, H]
+    const uint8_t* xs;                 // UE8M0 [R, H / 32] (not QUANT)
+    const int64_t* idx; const float* rw;
+    WMat w1, w3, w2;
+    const float* add; float* y;
+    uint32_t* hc;                      // [NBD][P][I / 4]  act-quantised intermediate, code words, one copy per column block
+    uint32_t* hsw;                     // [NBD][P][I / 32] its scales, one word each
+    float* yd;                         // [P][H] per-pair outputs
+    int* err;
+    int R, TT, topk, E, P, Gmax, H, I, NJ, NBD, nU;
+};
+
+__device__ __forceinline__ uint32_t ld_dev32(const void* p) { return __hip_atomic_load((const uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ uint64_t ld_dev64(const void* p) { return __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_dev32(void* p, uint32_t v) { __hip_atomic_store((uint32_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_dev64(void* p, uint64_t v) { __hip_atomic_store((uint64_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// a non-temporal load is not kept in the CU's L1: a poll reads the XCD's L2 every time
+__device__ __forceinline__ uint32_t ld_l2(const float* p)
+{
+    return __builtin_nontemporal_load((const __attribute__((address_space(1))) uint32_t*)(uintptr_t)p);
+}
+
+__device__ __forceinline__ int pair_expert(const MArgs& a, int p)
+{
+    const int r = p / a.TT, k = p % a.TT;
+    return k < a.topk ? (int)a.idx[(int64_t)r * a.topk + k] : a.E + (k - a.topk);
+}
+struct Group { int e, n; };
+// item g of the call (distinct experts in order of first appearance): expert and its pairs (ascending) in rows[]
+__device__ __forceinline__ Group find_item(const MArgs& a, int g, int* sidx, unsigned char* isf, int* rows, int* misc)
+{
+    const int P = a.P, tid = threadIdx.x;
+    if (a.R == 1) {
+        if (g >= P) return Group{0, 0};
+        if (tid == 0) rows[0] = g;
+        __syncthreads();
+        return Group{pair_expert(a, g), 1};
+    }
+    if (tid == 0) { misc[0] = -1; misc[1] = 0; }
+    for (int p = tid; p < P; p += NT) sidx[p] = pair_expert(a, p);
+    __syncthreads();
+    for (int p = tid; p < P; p += NT) {
+        const int e = sidx[p];
+        bool first = true;
+        for (int q = 0; q < p; ++q) first &= sidx[q] != e;
+        isf[p] = first;
+    }
+    __syncthreads();
+    for (int p = tid; p < P; p += NT)
+        if (isf[p]) {
+            int before = 0;
+            for (int q = 0; q < p; ++q) before += isf[q];
+            if (before == g) misc[0] = sidx[p];
+        }
+    __syncthreads();
+    const int e = misc[0];
+    if (e < 0) return Group{0, 0};
+    for (int p = tid; p < P; p += NT)
+        if (sidx[p] == e) {
+            int slot = 0;
+            for (int q = 0; q < p; ++q) slot += sidx[q] == e;
+            rows[slot] = p;
+            atomicAdd(&misc[1], 1);
+        }
+    __syncthreads();
+    return Group{e, misc[1]};
+}
+
+template <int LAYOUT, bool QUANT, bool LOCAL>
+__global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int sidx[PMAXF], rows[RMAX], comb[RMAX], misc[4];
+    __shared__ unsigned char isf[PMAXF];
+    __shared__ float amx[NW][16];
+    __shared__ __align__(16) uint32_t hbw[16][8];          // the block's 32 code bytes per item row
+    __shared__ uint32_t he[16];
+    float (*red)[4][4][64] = (float (*)[4][4][64])smem;    // [wave][tile][v][lane]
+    unsigned char* extra = smem + RED_BYTES;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, rg = lane >> 4;
+    const int bid = blockIdx.x;
+    const bool isU = bid < a.nU;
+    const int H = a.H, I = a.I;
+    if (isU) {
+        // ================================================================ stage 1
+        __builtin_amdgcn_s_setprio(2);
+        const int g = bid / a.NJ, jb = bid % a.NJ, j0 = jb * 32;
+        const Group grp = find_item(a, g, sidx, isf, rows, misc);
+        if (grp.n == 0) return;
+        const int steps = H >> 7, nkg = (steps + 3) >> 2;
+        // ---- the first K group of this wave's weight rows, then the activations of its K groups
+        v4i A[4][4];
+        uint32_t sa[4];
+        {
+            const int kg = min(wave, nkg - 1);
+            load_group<LAYOUT>(a.w1, grp.e, j0, kg, lane, A[0], sa[0]);
+            load_group<LAYOUT>(a.w1, grp.e, j0 + 16, kg, lane, A[1], sa[1]);
+            load_group<LAYOUT>(a.w3, grp.e, j0, kg, lane, A[2], sa[2]);
+            load_group<LAYOUT>(a.w3, grp.e, j0 + 16, kg, lane, A[3], sa[3]);
+        }
+        unsigned char* xql = extra;                        // [n][H] E4M3 codes of the item's token rows
+        unsigned char* xsl = extra + (size_t)a.R * H;      // [n][H / 32] scales
+        if (QUANT) {
+            // act_quant per 32 (reference engine-rs/src/ds41/ops.rs:26-35): 4 lanes x 8 elements per block
+            for (int kg = wave; kg < nkg; kg += NW)
+                for (int r = 0; r < grp.n; ++r) {
+                    const int k = kg * 512 + lane * 8;
+                    if (k < H) {
+                        const int tok = rows[r] / a.TT;
+                        const uint4 raw = *(const uint4*)((const uint16_t*)a.x + (int64_t)tok * H + k);
+                        const uint32_t rw4[4] = {raw.x, raw.y, raw.z, raw.w};
+                        float v[8];
+                        float am = 0.f;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            v[2 * i] = __uint_as_float(rw4[i] << 16); v[2 * i + 1] = __uint_as_float(rw4[i] & 0xffff0000u);
+                            am = fmaxf(am, fmaxf(fabsf(v[2 * i]), fabsf(v[2 * i + 1])));
+                        }
+                        am = fmaxf(am, lane_xor<1>(am, lane));
+                        am = fmaxf(am, lane_xor<2>(am, lane));
+                        const uint32_t e = aq_scale(am);
+                        uint32_t lo = 0, hi = 0;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { lo |= aq_byte(v[i], e) << (8 * i); hi |= aq_byte(v[4 + i], e) << (8 * i); }
+                        *(uint2*)(xql + (size_t)r * H + k) = make_uint2(lo, hi);
+                        if ((lane & 3) == 0) xsl[(size_t)r * (H >> 5) + (k >> 5)] = (unsigned char)e;
+                    }
+                }
+        }
+        const bool valid = c < grp.n;
+        const int rc = valid ? c : 0;
+        const int pair = rows[rc];
+        const uint8_t* xr = QUANT ? xql + (size_t)rc * H : (const uint8_t*)a.x + (int64_t)(pair / a.TT) * H;
+        const uint8_t* xsr = QUANT ? xsl + (size_t)rc * (H >> 5) : a.xs + (int64_t)(pair / a.TT) * (H >> 5);
+        v4f acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) { acc[t] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(acc[t])); }
+        for (int kg = wave; kg < nkg; kg += NW) {
+            if (kg != wave) {
+                load_group<LAYOUT>(a.w1, grp.e, j0, kg, lane, A[0], sa[0]);
+                load_group<LAYOUT>(a.w1, grp.e, j0 + 16, kg, lane, A[1], sa[1]);
+                load_group<LAYOUT>(a.w3, grp.e, j0, kg, lane, A[2], sa[2]);
+                load_group<LAYOUT>(a.w3, grp.e, j0 + 16, kg, lane, A[3], sa[3]);
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int step = kg * 4 + s;
+                if (step >= steps) break;
+                v8i b; uint32_t sb;
+                load_b(xr, xsr, step, lane, b, sb);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[t] = mfma_group_step(s, A[t][s], b, acc[t], sa[t], sb);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][t][v][lane] = acc[t][v];
+        __syncthreads();
+        // epilogue: thread (wave = (tp, v), lane = (c, rg)) owns feature j0 + 16 tp + 4 rg + v of column c
+        const int tp = wave >> 2, v = wave & 3;
+        float gsum = 0.f, usum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) { gsum += red[w][tp][v][lane]; usum += red[w][2 + tp][v][lane]; }
+        float wgt = 0.f;
+        if (valid) { const int k = pair % a.TT; wgt = k < a.topk ? a.rw[(int64_t)(pair / a.TT) * a.topk + k] : 1.0f; }
+        const float gt = fminf(bf16_round(gsum), 10.f);
+        const float up = fminf(fmaxf(bf16_round(usum), -10.f), 10.f);
+        const float yv = bf16_round(silu(gt) * up * wgt);
+        float am = fabsf(yv);
+        am = fmaxf(am, lane_xor<16>(am, lane));
+        am = fmaxf(am, lane_xor<32>(am, lane));
+        if (rg == 0) amx[wave][c] = am;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < NW; ++w) am = fmaxf(am, amx[w][c]);
+        const uint32_t e = aq_scale(am);
+        ((unsigned char*)hbw[c])[16 * tp + 4 * rg + v] = (unsigned char)aq_byte(yv, e);
+        if (wave == 0 && rg == 0) he[c] = e;
+        __syncthreads();
+        // ---- hand the rows' 32 codes + scale to every column block's copy of h (device-coherent: the readers sit on all XCDs)
+        const int per = grp.n * 9;
+        for (int u = tid; u < a.NBD * per; u += NT) {
+            const int q = u / per, rem = u % per, cc = rem / 9, w = rem % 9;
+            const int64_t row = (int64_t)q * a.P + rows[cc];
+            if (w < 8) {
+                uint32_t word = hbw[cc][w];
+                if (word == EMPTY) word = 0xffffff7fu;
+                st_dev32(a.hc + row * (I >> 2) + jb * 8 + w, word);
+            } else st_dev32(a.hsw + row * (I >> 5) + jb, he[cc]);
+        }
+        return;
+    }
+    // ==================================================================== stage 2
+    int nb = -1, g = 0;
+    {
+        const int b = bid - a.nU, xcd = b % NXCD, li = b / NXCD;
+        const int q = (li / a.Gmax) * NXCD + xcd;          // column block q lives on XCD q % 8
+        if (q < a.NBD) { nb = q; g = li % a.Gmax; }
+    }
+    if (nb < 0) return;
+    const Group grp = find_item(a, g, sidx, isf, rows, misc);
+    if (grp.n == 0) return;
+    const int sub = wave >> 2, kw = wave & 3;              // 32-column half of the block, K group within a round
+    const int n0 = nb * DC + sub * 32;
+    const int steps = I >> 7, nkg = (steps + 3) >> 2;
+    v4i A[2][4];
+    uint32_t sa[2];
+    {
+        const int kg = min(kw, nkg - 1);
+        load_group<LAYOUT>(a.w2, grp.e, n0, kg, lane, A[0], sa[0]);
+        load_group<LAYOUT>(a.w2, grp.e, n0 + 16, kg, lane, A[1], sa[1]);
+    }
+    // token rows of this item that this block sums: those whose other experts all belong to earlier items
+    if (a.R == 1) { if (tid == 0) comb[0] = g == a.P - 1; }
+    else {
+        if (tid < grp.n) comb[tid] = 1;
+        __syncthreads();
+        const int fo = rows[0];
+        for (int u = tid; u < grp.n * a.TT; u += NT) {
+            const int i = u / a.TT, k = u % a.TT, e = sidx[(rows[i] / a.TT) * a.TT + k];
+            bool seen = false;
+            for (int q = 0; q <= fo; ++q) seen |= sidx[q] == e;
+            if (!seen) comb[i] = 0;
+        }
+    }
+    if (tid == 0) misc[2] = 1;
+    __syncthreads();
+    // B operands of a round in LDS: [kw][step][g4][row < n] x (8 code words + 1 scale word), written by the waves of half 0
+    uint32_t* hl = (uint32_t*)extra;
+    const bool valid = c < grp.n;
+    const int rc = valid ? c : 0;
+    v4f acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) { acc[t] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(acc[t])); }
+    for (int rd = 0; rd * 4 < nkg; ++rd) {
+        const int kg = rd * 4 + kw;
+        const bool have = kg < nkg;
+        if (rd > 0) {
+            __syncthreads();                               // the previous round's operands have been read
+            if (have) {
+                load_group<LAYOUT>(a.w2, grp.e, n0, kg, lane, A[0], sa[0]);
+                load_group<LAYOUT>(a.w2, grp.e, n0 + 16, kg, lane, A[1], sa[1]);
+            }
+        }
+        if (sub == 0 && have) {
+            // cheap wait first (one scale word per 32-block of the K group, first row), then every word of this lane
+            const int nblk = min(16, (I >> 5) - kg * 16);
+            int spins = 0;
+            for (;;) {
+                const uint32_t v = lane < nblk ? ld_dev32(a.hsw + ((int64_t)nb * a.P + rows[0]) * (I >> 5) + kg * 16 + lane) : 0u;
+                if (__builtin_amdgcn_ballot_w64(v == EMPTY) == 0 || ++spins >= SPIN_MAX) break;
+                __builtin_amdgcn_s_sleep(4);
+            }
+            if (valid) {
+                const int64_t row = (int64_t)nb * a.P + rows[c];
+                uint32_t* pc = a.hc + row * (I >> 2);
+                uint32_t* ps = a.hsw + row * (I >> 5);
+                uint64_t w[4][4];
+                uint32_t sw[4];
+                bool ok = false;
+                for (spins = 0; spins < SPIN_MAX && !ok; ++spins) {
+                    ok = true;
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const int step = min(kg * 4 + s, steps - 1);
+                        w[s][0] = ld_dev64(pc + step * 32 + rg * 4); w[s][1] = ld_dev64(pc + step * 32 + rg * 4 + 2);
+                        w[s][2] = ld_dev64(pc + step * 32 + 16 + rg * 4); w[s][3] = ld_dev64(pc + step * 32 + 16 + rg * 4 + 2);
+                        sw[s] = ld_dev32(ps + step * 4 + rg);
+                    }
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        ok = ok && sw[s] != EMPTY;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) ok = ok && (uint32_t)w[s][i] != EMPTY && (uint32_t)(w[s][i] >> 32) != EMPTY;
+                    }
+                    if (!ok) __builtin_amdgcn_s_sleep(1);
+                }
+                if (!ok) misc[2] = 0;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const int step = kg * 4 + s;
+                    if (step < steps && ok) {
+                        st_dev64(pc + step * 32 + rg * 4, EMPTY2); st_dev64(pc + step * 32 + rg * 4 + 2, EMPTY2);
+                        st_dev64(pc + step * 32 + 16 + rg * 4, EMPTY2); st_dev64(pc + step * 32 + 16 + rg * 4 + 2, EMPTY2);
+                        st_dev32(ps + step * 4 + rg, EMPTY);
+                    }
+                    uint32_t* o = hl + (((kw * 4 + s) * 4 + rg) * RMAX + c) * 9;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { o[2 * i] = (uint32_t)w[s][i]; o[2 * i + 1] = (uint32_t)(w[s][i] >> 32); }
+                    o[8] = sw[s];
+                }
+            }
+        }
+        __syncthreads();
+        if (rd == 0) __builtin_amdgcn_s_setprio(3);        // from here on this block is the critical path
+        if (have && misc[2]) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int step = kg * 4 + s;
+                if (step >= steps) break;
+                const uint32_t* o = hl + (((kw * 4 + s) * 4 + rg) * RMAX + rc) * 9;
+                const v8i b = v8i{(int)o[0], (int)o[1], (int)o[2], (int)o[3], (int)o[4], (int)o[5], (int)o[6], (int)o[7]};
+                const uint32_t sb = o[8];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) acc[t] = mfma_group_step(s, A[t][s], b, acc[t], sa[t], sb);
+            }
+        }
+    }
+    if (!misc[2]) { if (tid == 0) atomicExch(a.err, 1); return; }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][t][v][lane] = acc[t][v];
+    __syncthreads();
+    // thread (wave = (sub, v), lane) sums element v of both tiles over the four K waves of its half, in wave order
+    if (valid) {
+        const int v = kw;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) s += red[sub * 4 + w][t][v][lane];
+            uint32_t u = __float_as_uint(s);
+            if (u == EMPTY) u = 0x7fc00000u;
+            float* p = a.yd + (int64_t)rows[c] * H + n0 + 16 * t + 4 * rg + v;
+            if (LOCAL) *(uint32_t*)p = u; else st_dev32(p, u);
+        }
+    }
+    // ---- the token rows this block sums: wave i takes item row i, lane = column
+    if (wave < grp.n && comb[wave]) {
+        const int tok = rows[wave] / a.TT, col = nb * DC + lane;
+        const float base = a.add ? a.add[(int64_t)tok * H + col] : 0.f;
+        float* py[TTMAX];
+#pragma unroll
+        for (int k = 0; k < TTMAX; ++k) py[k] = a.yd + (int64_t)(tok * a.TT + (k < a.TT ? k : 0)) * H + col;
+        uint32_t o[TTMAX];
+        int spins = 0;
+        bool ok;
+        for (;;) {
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int k = 0; k < TTMAX; ++k) o[k] = LOCAL ? ld_l2(py[k]) : ld_dev32(py[k]);
+            ok = true;
+#pragma unroll
+            for (int k = 0; k < TTMAX; ++k) ok = ok && o[k] != EMPTY;
+            if (__builtin_amdgcn_ballot_w64(!ok) == 0) { ok = true; break; }
+            if (++spins >= SPIN_MAX) { ok = false; break; }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        if (ok) {
+#pragma unroll
+            for (int k = 0; k < TTMAX; ++k) { if (LOCAL) *(uint32_t*)py[k] = EMPTY; else st_dev32(py[k], EMPTY); }
+            float accs = base;                             // add + shared experts, then the routed experts in slot order
+#pragma unroll
+            for (int k = 0; k < TTMAX; ++k) if (k >= a.topk && k < a.TT) accs += __uint_as_float(o[k]);
+            float s = 0.f;
+#pragma unroll
+            for (int k = 0; k < TTMAX; ++k) if (k < a.topk) s += __uint_as_float(o[k]);
+            a.y[(int64_t)tok * H + col] = accs + s;
+        } else if (lane == 0) atomicExch(a.err, 1);
+    }
+}
+
+__global__ void fill_kernel(uint32_t* p, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = i < HEAD / 4 ? 0u : EMPTY;
+}
+
+struct FPlan { int TT, ET, P, Gmax, NJ, NBD, nU, nD; size_t hc, hsw, yd, total, lds; };
+FPlan fplan(int R, int H, int I, int topk, int E, int n_shared)
+{
+    FPlan p;
+    p.TT = topk + n_shared; p.ET = E + n_shared;
+    p.P = R * p.TT;
+    p.Gmax = p.P < p.ET ? p.P : p.ET;
+    p.NJ = I / 32; p.NBD = H / DC;
+    p.nU = p.Gmax * p.NJ;
+    p.nD = (p.NBD + NXCD - 1) / NXCD * NXCD * p.Gmax;
+    size_t o = HEAD;
+    auto take = [&](size_t n) { const size_t q = o; o += align256(n); return q; };
+    p.hc = take((size_t)p.NBD * p.P * I);
+    p.hsw = take((size_t)p.NBD * p.P * (I / 32) * 4);
+    p.yd = take((size_t)p.P * H * 4);
+    p.total = o;
+    const size_t lu = (size_t)R * H + (size_t)R * (H / 32), ld = (size_t)16 * 4 * RMAX * 9 * 4;
+    p.lds = RED_BYTES + ((lu > ld ? lu : ld) + 15) / 16 * 16;
+    return p;
+}
+
+int g_local = -1;
+__global__ void xcd_probe_kernel(int* out)
+{
+    if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((31 << 11) | 20) & 0xf;
+}
+
+template <int LAYOUT, bool QUANT>
+int launch(const MArgs& a, const FPlan& p, hipStream_t st)
+{
+    const dim3 grid(p.nU + p.nD), blk(NT);
+    if (g_local == 1) {
+        static bool attr = false;
+        if (!attr) { (void)hipFuncSetAttribute((const void*)mx_fused_kernel<LAYOUT, QUANT, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); attr = true; }
+        mx_fused_kernel<LAYOUT, QUANT, true><<<grid, blk, p.lds, st>>>(a);
+    } else {
+        static bool attr = false;
+        if (!attr) { (void)hipFuncSetAttribute((const void*)mx_fused_kernel<LAYOUT, QUANT, false>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); attr = true; }
+        mx_fused_kernel<LAYOUT, QUANT, false><<<grid, blk, p.lds, st>>>(a);
+    }
+    return launch_status();
+}
+
+}  // namespace
+
+bool mx_fused_ok(int R, int H, int I, int topk, int E, int n_shared)
+{
+    if (R < 1 || R > RMAX || topk + n_shared > TTMAX || H % DC || I % 128 || H % 128) return false;
+    const FPlan p = fplan(R, H, I, topk, E, n_shared);
+    return p.lds <= 96 * 1024;
+}
+size_t mx_fused_ws_bytes(int R, int H, int I, int topk, int E, int n_shared) { return fplan(R, H, I, topk, E, n_shared).total; }
+
+// Checks once per process that workgroup b of a 1-D grid runs on XCD b % 8 (synchronises: not for use under stream capture).
+int mx_xcd_probe()
+{
+    if (g_local >= 0) return g_local;
+    constexpr int NB = 1024;
+    int* d = nullptr;
+    if (hipMalloc(&d, NB * sizeof(int)) != hipSuccess) return g_local = 0;
+    xcd_probe_kernel<<<NB, 64>>>(d);
+    int h[NB];
+    const bool copied = hipMemcpy(h, d, sizeof(h), hipMemcpyDeviceToHost) == hipSuccess;
+    (void)hipFree(d);
+    bool ok = copied;
+    for (int i = 0; ok && i < NB; ++i) ok = h[i] == h[i % NXCD];
+    for (int i = 0; ok && i < NXCD; ++i)
+        for (int j = 0; j < i; ++j) ok = ok && h[i] != h[j];
+    return g_local = ok ? 1 : 0;
+}
+
+// every exchanged word of a workspace idle, its error flag clear
+int mx_fused_ws_prepare(void* ws, size_t bytes, hipStream_t st)
+{
+    const int64_t n = (int64_t)(bytes / 4);
+    if (n > 0) fill_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((uint32_t*)ws, n);
+    return launch_status();
+}
+
+// x: bf16 [R, H] when xs == nullptr (quantised inside), else E4M3 [R, H] with scales xs.  clean = the workspace is idle
+// (prepared once and only used by this path since).
+int mx_fused_launch(const void* x, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3, const void* s3,
+                    const void* w2, const void* s2, int layout, int H, int I, int topk, int E, int n_shared, const float* add, float* y, void* ws, int clean,
+                    hipStream_t st)
+{
+    const FPlan p = fplan(R, H, I, topk, E, n_shared);
+    char* b = (char*)ws;
+    MArgs a;
+    a.x = x; a.xs = (const uint8_t*)xs; a.idx = idx; a.rw = rw;
+    a.w1 = WMat{(const uint8_t*)w1, (const uint8_t*)s1, I, H}; a.w3 = WMat{(const uint8_t*)w3, (const uint8_t*)s3, I, H};
+    a.w2 = WMat{(const uint8_t*)w2, (const uint8_t*)s2, H, I};
+    a.add = add; a.y = y;
+    a.hc = (uint32_t*)(b + p.hc); a.hsw = (uint32_t*)(b + p.hsw); a.yd = (float*)(b + p.yd); a.err = (int*)b;
+    a.R = R; a.TT = p.TT; a.topk = topk; a.E = E; a.P = p.P; a.Gmax = p.Gmax; a.H = H; a.I = I; a.NJ = p.NJ; a.NBD = p.NBD; a.nU = p.nU;
+    if (!clean) {
+        const int rc = mx_fused_ws_prepare(ws, p.total, st);
+        if (rc) return rc;
+    }
+    const bool quant = xs == nullptr;
+    switch (layout) {
+        case L_T16: return quant ? launch<L_T16, true>(a, p, st) : launch<L_T16, false>(a, p, st);
+        case L_NATURAL: return quant ? launch<L_NATURAL, true>(a, p, st) : launch<L_NATURAL, false>(a, p, st);
+        case L_PACK8: return quant ? launch<L_PACK8, true>(a, p, st) : launch<L_PACK8, false>(a, p, st);
+        case L_MX8: return quant ? launch<L_MX8, true>(a, p, st) : launch<L_MX8, false>(a, p, st);
+    }
+    return 1;
+}
+
+}  // namespace mx
+}  // namespace spk

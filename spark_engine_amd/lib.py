@@ -46,6 +46,8 @@ SIGNATURES = {
     "spark_mxfp4_moe_ws_bytes": (sz, [i32, i32, i32, i32, i32, i32]),
     "spark_mxfp4_moe_q": (i32, [vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp]),
     "spark_mxfp4_moe": (i32, [vp, vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp]),
+    "spark_mxfp4_moe_ws_init": (i32, [vp, sz, vp]),
+    "spark_mxfp4_moe_x": (i32, [vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp, vp, vp, i32, vp]),
     "ds41_moe_mx_set_s2": (None, [i32]), "ds41_moe_mx_get_s2": (i32, []), "ds41_moe_gr16_max": (None, [i32]),
     "ds41_moe_mx_col_passes": (i32, [i32, i32, i32]), "ds41_moe_mx_pair_b16": (i32, [i32, i32, i32]),
     "ds41_moe_mx_ws_bytes": (sz, [i32, i32, i32, i32]), "ds41_moe_ws_bytes": (sz, [i32, i32, i32, i32]),

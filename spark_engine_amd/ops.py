@@ -235,6 +235,34 @@ def mxfp4_moe(x, idx, rw, ex, add=None, y=None, ws=None, scratch=None, natural=F
     return y
 
 
+def mxfp4_moe_ws_alloc(R, ex, topk, device="cuda:0"):
+    """A workspace prepared once (spark_mxfp4_moe_ws_init): calls of mxfp4_moe_x with ws_clean=True then run as one launch."""
+    ws = torch.empty(mxfp4_moe_ws(R, ex, topk), dtype=torch.uint8, device=device)
+    _ck(_lib().spark_mxfp4_moe_ws_init(_p(ws), ws.numel(), _st()), "spark_mxfp4_moe_ws_init")
+    return ws
+
+
+def mxfp4_moe_x(x, idx, rw, ex, xs=None, add=None, y=None, ws=None, ws_clean=False, multi_kernel=False, natural=False):
+    """The decode entry (R <= 8): x bf16 [R, H] (quantised inside the kernel) or E4M3 bytes with scales xs -> y f32 [R, H]."""
+    R, H = x.shape
+    topk = idx.shape[1]
+    dev = x.device
+    if y is None:
+        y = torch.empty(R, H, dtype=torch.float32, device=dev)
+    if ws is None:
+        ws = torch.empty(mxfp4_moe_ws(R, ex, topk), dtype=torch.uint8, device=dev)
+        ws_clean = False
+    if natural:
+        w1, s1, w3, s3, w2, s2 = ex.natural
+        layout = 1
+    else:
+        (w1, w3, w2), (s1, s3, s2), layout = ex.packed, (None, None, None), 0
+    flags = (1 if ws_clean else 0) | (2 if multi_kernel else 0)
+    _ck(_lib().spark_mxfp4_moe_x(_p(_dev(x)), _p(xs), R, _p(_dev(idx)), _p(_dev(rw)), _p(w1), _p(s1), _p(w3), _p(s3), _p(w2), _p(s2),
+                                 layout, H, ex.I, topk, ex.E, ex.n_shared, _p(add), _p(y), _p(ws), flags, _st()), "spark_mxfp4_moe_x")
+    return y
+
+
 # reference tile layouts (kern.rs:718-734), restated with tensor view/permute exactly as the Rust does
 def moe_pack(w, s):
     e, rows, kb = w.shape

@@ -64,6 +64,29 @@ def test_moe_zero_codes_give_add(ops):
     assert np.array_equal(host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex, add=dev(add))), add)
 
 
+@pytest.mark.parametrize("R,H,I,E,topk,ns", [(1, 1024, 512, 12, 6, 1), (2, 512, 384, 6, 3, 1), (4, 1024, 256, 5, 2, 2), (8, 512, 256, 4, 2, 0)])
+def test_single_launch_equals_several_kernel_path_bitwise(ops, oracle, R, H, I, E, topk, ns):
+    # the decode entry runs the whole layer as one launch with the same summation orders as the several-kernel path;
+    # a prepared workspace is reused call after call (the exchanged words clear themselves)
+    g = synth.rng(230 + R)
+    ws, x, idx, rw = _case(g, R, H, I, E, topk, ns)
+    ex = ops.Mxfp4Experts(*[dev(a) for a in ws], n_shared=ns)
+    wsd = ops.mxfp4_moe_ws_alloc(R, ex, topk)
+    for it in range(3):
+        x = synth.randn_bf16(g, (R, H))
+        idx = np.stack([g.permutation(E)[:topk] for _ in range(R)]).astype(np.int64)
+        add = g.standard_normal((R, H)).astype(np.float32)
+        ref = oracle.mxfp4_moe(x, idx, rw, *ws, n_shared=ns, add=add)
+        one = host(ops.mxfp4_moe_x(dev_bf16(x), dev(idx), dev(rw), ex, add=dev(add), ws=wsd, ws_clean=True))
+        assert rel_l2(one, ref) <= TOL, rel_l2(one, ref)
+        xq, xs = ops.act_quant_fp8(dev_bf16(x))
+        several = host(ops.mxfp4_moe_x(xq, dev(idx), dev(rw), ex, xs=xs, add=dev(add), multi_kernel=True))
+        assert np.array_equal(one, several)
+        given = host(ops.mxfp4_moe_x(xq, dev(idx), dev(rw), ex, xs=xs, add=dev(add), ws=wsd, ws_clean=True))   # activations quantised by the caller
+        assert np.array_equal(one, given)
+    assert int(wsd.view(torch.int32)[0].item()) == 0                  # no wait expired
+
+
 def test_moe_many_rows_multi_column_groups(ops, oracle):
     # more than 16 rows on one expert: several MFMA column groups per item, items of 64 rows
     g = synth.rng(212)
