@@ -71,12 +71,6 @@ __device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
 // ---- wave64 cross-lane primitives ----
 // value of lane (lane ^ mask) for mask < 64
 __device__ __forceinline__ float xor_f(float v, int mask) { return __shfl_xor(v, mask, 64); }
-__device__ __forceinline__ float wave_sum(float v)
-{
-#pragma unroll
-    for (int o = 32; o; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
 __device__ __forceinline__ float wave_max(float v)
 {
 #pragma unroll
@@ -106,6 +100,14 @@ template <int M> __device__ __forceinline__ float lane_xor(float v, int lane)
         const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
         return __uint_as_float((lane & 32) ? r[0] : r[1]);
     }
+}
+// butterfly sum over the wave, partners 32, 16, ..., 1 apart in that order (every lane ends with the total)
+__device__ __forceinline__ float wave_sum(float v)
+{
+    const int lane = threadIdx.x & 63;
+    v += lane_xor<32>(v, lane); v += lane_xor<16>(v, lane); v += lane_xor<8>(v, lane);
+    v += lane_xor<4>(v, lane); v += lane_xor<2>(v, lane); v += lane_xor<1>(v, lane);
+    return v;
 }
 template <int M> __device__ __forceinline__ void fwht_stage(float& v0, float& v1, int lane)
 {

@@ -8,6 +8,7 @@
 // products in binary32 with v_dot2_f32_bf16; the block scale multiplies the piece's partial sum; lanes are summed with
 // a butterfly.  Activations are staged once per workgroup in LDS.
 #include "common.hpp"
+#include <type_traits>
 
 using namespace spk;
 
@@ -15,7 +16,7 @@ typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
 
 namespace {
 
-constexpr int GEMV_WAVES = 4, RPW = 4;
+constexpr int GEMV_WAVES = 4, RPW = 4, UNR = 4;
 
 __device__ __forceinline__ bf2 as_bf2(uint32_t v) { bf2 r; __builtin_memcpy(&r, &v, 4); return r; }
 
@@ -42,9 +43,7 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void qgemv_kernel(const uint16_t* 
     const int wg_row0 = blockIdx.x * (GEMV_WAVES * RPW);
     // grouped (block-diagonal) weights read input group row / rpg; a workgroup's rows share the group (rpg % 32 == 0)
     const int64_t xoff = rpg ? (int64_t)(wg_row0 / rpg) * k : 0;
-    stage_x(x, xs, xoff, xl, m, k);
     const int row0 = wg_row0 + wave * RPW;
-    if (row0 >= n) return;
     constexpr int EPP = FMT == 0 ? 32 : 16;               // elements per 16-byte piece
     const int64_t rb = FMT == 0 ? k / 2 : k;              // bytes per weight row
     float acc[RPW][M];
@@ -52,49 +51,78 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void qgemv_kernel(const uint16_t* 
     for (int i = 0; i < RPW; ++i)
 #pragma unroll
         for (int r = 0; r < M; ++r) acc[i][r] = 0.f;
-    for (int c = lane * EPP; c < k; c += 64 * EPP) {
-        uint4 p[RPW];
-        float s[RPW];
+    // one step = the lane's 16-byte piece of each of the wave's RPW rows; NS steps are loaded together
+    auto load_steps = [&](auto ns, int c0, uint4 (&p)[UNR][RPW], float (&s)[UNR][RPW]) {
 #pragma unroll
-        for (int i = 0; i < RPW; ++i) {
-            const int row = row0 + i < n ? row0 + i : n - 1;
-            p[i] = ld_stream16(w + (int64_t)row * rb + (FMT == 0 ? c / 2 : c));
-            if (FMT == 0) s[i] = e8m0_to_f32(((const uint8_t*)sc)[(int64_t)row * (k >> 5) + (c >> 5)]);
-            else if (FMT == 1) s[i] = e8m0_to_f32(((const uint8_t*)sc)[(int64_t)(row >> 5) * (k >> 5) + (c >> 5)]);
-            else s[i] = ((const float*)sc)[(int64_t)(row / bs) * ((k + bs - 1) / bs) + c / bs];
-        }
+        for (int u = 0; u < decltype(ns)::value; ++u) {
+            const int c = c0 + u * 64 * EPP;
 #pragma unroll
-        for (int i = 0; i < RPW; ++i) {
-            const uint32_t pw[4] = {p[i].x, p[i].y, p[i].z, p[i].w};
-            bf2 wv[EPP / 2];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if (FMT == 0) {
-                    wv[4 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 0);
-                    wv[4 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 1);
-                    wv[4 * j + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 2);
-                    wv[4 * j + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 3);
-                } else {
-                    wv[2 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, false);
-                    wv[2 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, true);
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < M; ++r) {
-                if (r >= m) break;
-                const uint32_t* xp = (const uint32_t*)(xl + r * k + c);
-                float t = 0.f;
-#pragma unroll
-                for (int j = 0; j < EPP / 2; j += 4) {
-                    const uint4 xv = *(const uint4*)(xp + j);
-                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 0], as_bf2(xv.x), t, false);
-                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 1], as_bf2(xv.y), t, false);
-                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 2], as_bf2(xv.z), t, false);
-                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 3], as_bf2(xv.w), t, false);
-                }
-                acc[i][r] = __builtin_fmaf(t, s[i], acc[i][r]);
+            for (int i = 0; i < RPW; ++i) {
+                const int row = row0 + i < n ? row0 + i : n - 1;
+                p[u][i] = ld_stream16(w + (int64_t)row * rb + (FMT == 0 ? c / 2 : c));
+                if (FMT == 0) s[u][i] = e8m0_to_f32(((const uint8_t*)sc)[(int64_t)row * (k >> 5) + (c >> 5)]);
+                else if (FMT == 1) s[u][i] = e8m0_to_f32(((const uint8_t*)sc)[(int64_t)(row >> 5) * (k >> 5) + (c >> 5)]);
+                else s[u][i] = ((const float*)sc)[(int64_t)(row / bs) * ((k + bs - 1) / bs) + c / bs];
             }
         }
+    };
+    auto mul_steps = [&](auto ns, int c0, const uint4 (&p)[UNR][RPW], const float (&s)[UNR][RPW]) {
+#pragma unroll
+        for (int u = 0; u < decltype(ns)::value; ++u) {
+            const int c = c0 + u * 64 * EPP;
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) {
+                const uint32_t pw[4] = {p[u][i].x, p[u][i].y, p[u][i].z, p[u][i].w};
+                bf2 wv[EPP / 2];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (FMT == 0) {
+                        wv[4 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 0);
+                        wv[4 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 1);
+                        wv[4 * j + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 2);
+                        wv[4 * j + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 3);
+                    } else {
+                        wv[2 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, false);
+                        wv[2 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, true);
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < M; ++r) {
+                    if (r >= m) break;
+                    const uint32_t* xp = (const uint32_t*)(xl + r * k + c);
+                    float t = 0.f;
+#pragma unroll
+                    for (int j = 0; j < EPP / 2; j += 4) {
+                        const uint4 xv = *(const uint4*)(xp + j);
+                        t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 0], as_bf2(xv.x), t, false);
+                        t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 1], as_bf2(xv.y), t, false);
+                        t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 2], as_bf2(xv.z), t, false);
+                        t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 3], as_bf2(xv.w), t, false);
+                    }
+                    acc[i][r] = __builtin_fmaf(t, s[u][i], acc[i][r]);
+                }
+            }
+        }
+    };
+    uint4 p[UNR][RPW];
+    float s[UNR][RPW];
+    constexpr int BATCH = UNR * 64 * EPP;                 // columns of a full batch of steps
+    int c = lane * EPP;
+    const bool active = row0 < n;
+    // the first batch is on its way before the activations are staged (every wave of the workgroup takes part in the staging)
+    const bool first_full = c + (UNR - 1) * 64 * EPP < k;  // same for every lane when k is a multiple of 64 * EPP, else the lanes past the end go stepwise
+    const bool go = active && __builtin_amdgcn_ballot_w64(!first_full) == 0;
+    if (go) load_steps(std::integral_constant<int, UNR>{}, c, p, s);
+    stage_x(x, xs, xoff, xl, m, k);
+    if (!active) return;
+    if (go) { mul_steps(std::integral_constant<int, UNR>{}, c, p, s); c += BATCH; }
+    for (; __builtin_amdgcn_ballot_w64(c + (UNR - 1) * 64 * EPP >= k) == 0; c += BATCH) {
+        load_steps(std::integral_constant<int, UNR>{}, c, p, s);
+        mul_steps(std::integral_constant<int, UNR>{}, c, p, s);
+    }
+    for (; c < k; c += 64 * EPP) {
+        load_steps(std::integral_constant<int, 1>{}, c, p, s);
+        mul_steps(std::integral_constant<int, 1>{}, c, p, s);
     }
 #pragma unroll
     for (int i = 0; i < RPW; ++i)
