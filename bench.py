@@ -21,6 +21,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+FP8_PEAK_TFLOPS = 5000.0       # MI355X published dense FP8 matrix rate (the block-scaled FP8 x FP4 products run at it)
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known
 # size); filled in from the committed counter summaries, None where no counter run exists
 TRAFFIC = {("c2", 1): 17397800}
@@ -32,7 +33,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=640)
     ap.add_argument("--warmup", type=int, default=128)
     ap.add_argument("--batch", type=int, default=1, help="tokens per step of the headline workload (1 or 4)")
-    ap.add_argument("--config", default="c2", choices=["c2", "c3", "c4a", "c4b"],
+    ap.add_argument("--config", default="c2", choices=["c2", "c3", "c4a", "c4b", "c5"],
                     help="headline workload: c2 EXL3 MoE (default, the metric's configuration), c3 MXFP4 MoE, c4a/c4b FP8 dense 7168x4096 / 4096x7168")
     ap.add_argument("--only-headline", action="store_true", help="skip the other configurations' lines")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -159,6 +160,38 @@ class Mxfp4Layer:
         return d * self.BYTES_PER_EXPERT + self.R * self.H * (2 + 4), float(d)
 
 
+class Mxfp4Prefill(Mxfp4Layer):
+    """Config 5: the MXFP4 layer at prefill size: 2048 tokens, top-6 of 384 experts drawn Zipf(1.1), no shared expert.  The routes are
+    inputs here (drawn on the host, as the configuration prescribes); a step = act_quant + grouped gate/up/down + weighted sum."""
+    NS = 0
+
+    def __init__(self, torch, ops, R, inst, seed=3):
+        from spark_engine_amd import synth
+        super().__init__(torch, ops, R, inst, seed)
+        g = synth.rng(seed)
+        for k in range(inst):
+            idx, w = synth.zipf_routes(g, R, self.E, self.TOPK)
+            self.idx[k].copy_(torch.from_numpy(idx)); self.rw[k].copy_(torch.from_numpy(w))
+        self.ws = torch.empty(ops.mxfp4_moe_ws(R, self.ex, self.TOPK), dtype=torch.uint8, device="cuda:0")
+        self.scratch = (torch.empty(R, self.H, dtype=torch.uint8, device="cuda:0"), torch.empty(R, self.H // 32, dtype=torch.uint8, device="cuda:0"))
+        self.name = f"C5 prefill-sized MXFP4 grouped GEMM (H {self.H}, I {self.I}, {self.E} experts top-{self.TOPK}, Zipf(1.1) routing), {R} tokens"
+        self.flops = 2.0 * R * self.TOPK * 3 * self.H * self.I
+
+    def step(self, i):
+        k = i % self.inst
+        self.ops.mxfp4_moe(self.x, self.idx[k], self.rw[k], self.ex, y=self.y[k], ws=self.ws, scratch=self.scratch)
+
+    dominant = None
+
+    def bytes_per_step(self):
+        idx = self.idx.cpu().numpy()
+        d = np.mean([len(set(idx[k].ravel().tolist())) for k in range(self.inst)])
+        P = self.R * self.TOPK
+        # weights of the distinct experts once + x in, h out and in (codes + scales), per-pair outputs out and in, y out
+        act = self.R * self.H * 2 + 2 * P * (self.I + self.I // 32) + 2 * P * self.H * 4 + self.R * self.H * 4
+        return d * self.BYTES_PER_EXPERT + act, float(d)
+
+
 class Fp8Dense:
     """Config 4: FP8 E4M3 dense projection with 128x128 FP32 block scales."""
     LAYERS = 1
@@ -225,9 +258,14 @@ def line_for(wl, ms):
     by, d = wl.bytes_per_step()
     us = ms * 1e3
     gbs = by / (us * 1e-6) / 1e9
-    return {"workload": wl.name, "us_per_layer": round(us, 3), "algorithmic_bytes": int(by), "distinct_experts": round(d, 2),
-            "achieved_GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
-            "tok_per_s_equiv": round(1e6 / (us * wl.LAYERS) * wl.R, 1), "layers_assumed": wl.LAYERS}
+    out = {"workload": wl.name, "us_per_layer": round(us, 3), "algorithmic_bytes": int(by), "distinct_experts": round(d, 2),
+           "achieved_GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+           "tok_per_s_equiv": round(1e6 / (us * wl.LAYERS) * wl.R, 1), "layers_assumed": wl.LAYERS}
+    if hasattr(wl, "flops"):                               # the contraction-sized configuration: matrix-unit rate next to the bandwidth
+        tf = wl.flops / (us * 1e-6) / 1e12
+        out.update({"flops": wl.flops, "achieved_TFLOPs": round(tf, 1), "frac_of_fp8_mfma_peak": round(tf / FP8_PEAK_TFLOPS, 4),
+                    "time_at_hbm_peak_us": round(by / (HBM_PEAK_GBS * 1e9) * 1e6, 1), "time_at_mfma_peak_us": round(wl.flops / (FP8_PEAK_TFLOPS * 1e12) * 1e6, 1)})
+    return out
 
 
 def main():
@@ -255,12 +293,15 @@ def main():
         wl = Exl3Layer(torch, ops, a.batch, INST)
     elif a.config == "c3":
         wl = Mxfp4Layer(torch, ops, a.batch, INST)
+    elif a.config == "c5":
+        INST = 4
+        wl = Mxfp4Prefill(torch, ops, 2048, INST)
     else:
         wl = Fp8Dense(torch, ops, a.batch, INST, *((7168, 4096) if a.config == "c4a" else (4096, 7168)))
     ms = time_steps(torch, wl, a.steps, a.warmup, INST)
     head = line_for(wl, ms)
     # the dominant kernel alone, same graphs and events: its average launch duration prices the roofline
-    if hasattr(wl, "dominant"):
+    if getattr(wl, "dominant", None) is not None:
         k_us = time_steps(torch, wl, a.steps, a.warmup, INST, wl.dominant) * 1e3
         k_name = wl.DOMINANT
     else:

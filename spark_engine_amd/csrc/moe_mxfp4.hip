@@ -102,6 +102,17 @@ __global__ __launch_bounds__(64 * UP_WAVES) void up_kernel(const uint8_t* __rest
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, rg = lane >> 4;
     const int j0 = blockIdx.x * 32;
     const int steps = H >> 7, nkg = (steps + 3) >> 2;
+    // a wave with one K group keeps its weight rows in registers for every group of 16 item rows: an item's weights are
+    // streamed once however many token rows it has
+    const bool resident = nkg <= UP_WAVES;
+    v4i a[4][4];
+    uint32_t sa[4];
+    if (resident && wave < nkg) {
+        load_group<LAYOUT>(w1, it.e, j0, wave, lane, a[0], sa[0]);
+        load_group<LAYOUT>(w1, it.e, j0 + 16, wave, lane, a[1], sa[1]);
+        load_group<LAYOUT>(w3, it.e, j0, wave, lane, a[2], sa[2]);
+        load_group<LAYOUT>(w3, it.e, j0 + 16, wave, lane, a[3], sa[3]);
+    }
     for (int cg = 0; cg * 16 < it.n; ++cg) {
         const int rr = cg * 16 + c;                // compact row of this lane's column within the item
         const bool valid = rr < it.n;
@@ -113,12 +124,12 @@ __global__ __launch_bounds__(64 * UP_WAVES) void up_kernel(const uint8_t* __rest
 #pragma unroll
         for (int t = 0; t < 4; ++t) { acc[t] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(acc[t])); }
         for (int kg = wave; kg < nkg; kg += UP_WAVES) {
-            v4i a[4][4];
-            uint32_t sa[4];
-            load_group<LAYOUT>(w1, it.e, j0, kg, lane, a[0], sa[0]);
-            load_group<LAYOUT>(w1, it.e, j0 + 16, kg, lane, a[1], sa[1]);
-            load_group<LAYOUT>(w3, it.e, j0, kg, lane, a[2], sa[2]);
-            load_group<LAYOUT>(w3, it.e, j0 + 16, kg, lane, a[3], sa[3]);
+            if (!resident) {
+                load_group<LAYOUT>(w1, it.e, j0, kg, lane, a[0], sa[0]);
+                load_group<LAYOUT>(w1, it.e, j0 + 16, kg, lane, a[1], sa[1]);
+                load_group<LAYOUT>(w3, it.e, j0, kg, lane, a[2], sa[2]);
+                load_group<LAYOUT>(w3, it.e, j0 + 16, kg, lane, a[3], sa[3]);
+            }
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 const int step = kg * 4 + s;
@@ -171,6 +182,13 @@ __global__ __launch_bounds__(64 * DN_WAVES) void down_kernel(const uint8_t* __re
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15;
     const int n0 = blockIdx.x * 32;
     const int steps = I >> 7, nkg = (steps + 3) >> 2;
+    const bool resident = nkg <= DN_WAVES;         // one K group per wave: its weight rows stay in registers for all item rows
+    v4i a[2][4];
+    uint32_t sa[2];
+    if (resident && wave < nkg) {
+        load_group<LAYOUT>(w2, it.e, n0, wave, lane, a[0], sa[0]);
+        load_group<LAYOUT>(w2, it.e, n0 + 16, wave, lane, a[1], sa[1]);
+    }
     for (int cg = 0; cg * 16 < it.n; ++cg) {
         const int rr = cg * 16 + c;
         const int pos = it.off + (rr < it.n ? rr : 0);
@@ -180,10 +198,10 @@ __global__ __launch_bounds__(64 * DN_WAVES) void down_kernel(const uint8_t* __re
 #pragma unroll
         for (int t = 0; t < 2; ++t) { acc[t] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(acc[t])); }
         for (int kg = wave; kg < nkg; kg += DN_WAVES) {
-            v4i a[2][4];
-            uint32_t sa[2];
-            load_group<LAYOUT>(w2, it.e, n0, kg, lane, a[0], sa[0]);
-            load_group<LAYOUT>(w2, it.e, n0 + 16, kg, lane, a[1], sa[1]);
+            if (!resident) {
+                load_group<LAYOUT>(w2, it.e, n0, kg, lane, a[0], sa[0]);
+                load_group<LAYOUT>(w2, it.e, n0 + 16, kg, lane, a[1], sa[1]);
+            }
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 const int step = kg * 4 + s;
@@ -264,7 +282,9 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
 }
 
 // ---------------------------------------------------------------- host side
-inline int gr_of(int R) { return R <= 16 ? 16 : 64; }
+// rows per item: 16 for decode sizes, up to 512 rows of an expert beyond (one pass over the expert's weights per item, which
+// stay in registers while the item's rows go by)
+inline int gr_of(int R) { return R <= 16 ? 16 : 512; }
 inline int gmax_of(int R, int TT, int ET)
 {
     const int64_t P = (int64_t)R * TT;
