@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 FP8_PEAK_TFLOPS = 5000.0       # MI355X published dense FP8 matrix rate (the block-scaled FP8 x FP4 products run at it)
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known
 # size); filled in from the committed counter summaries, None where no counter run exists
-TRAFFIC = {("c2", 1): 17397800}
+TRAFFIC = {("c2", 1): 18382700, ("c3", 1): 99397300}
 
 
 def parse():
@@ -323,9 +323,11 @@ def main():
         todo = [lambda: Exl3Layer(torch, ops, 4 if a.batch == 1 else 1, INST)]
         todo += [lambda R=R: Mxfp4Layer(torch, ops, R, INST) for R in (1, 2, 4)]
         todo += [lambda R=R, N=N, K=K: Fp8Dense(torch, ops, R, INST, N, K) for (N, K) in ((7168, 4096), (4096, 7168)) for R in (1, 4)]
+        todo += [lambda: Mxfp4Prefill(torch, ops, 2048, 4)]
         for mk in todo:
             w2 = mk()
-            others.append(line_for(w2, time_steps(torch, w2, 256, 64, INST)))
+            big = isinstance(w2, Mxfp4Prefill)
+            others.append(line_for(w2, time_steps(torch, w2, 32 if big else 256, 8 if big else 64, w2.inst)))
             del w2
             torch.cuda.empty_cache()
 

@@ -88,6 +88,8 @@ SPARK_API int ds41_mxfp4_gemv(const void* x, const void* w, const void* ws, floa
  * weight (0 = one matrix).  Replaces engine-rs/shim/ds41.cu:28-73,240,248. */
 SPARK_API int ds41_fp8_gemv_ex(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, int xs, int rpg, hipStream_t st);
 SPARK_API int ds41_fp8_gemv(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, hipStream_t st);
+/* The same product for up to 16 rows.  Replaces engine-rs/shim/ds41_mx.cu:1385-1393 (ds41_fp8_gemv_bx). */
+SPARK_API int ds41_fp8_gemv_bx(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, int xs, int rpg, hipStream_t st);
 /* w [n, k] E4M3 with fp32 scales [ceil(n/128), ceil(k/128)]; the projection of reference/ds41/kernel.py:96-119 (fp8_gemm) with bf16
  * activations used as given. */
 SPARK_API int spark_fp8_block128_gemv(const void* x, const void* w, const float* scales, float* y, int m, int n, int k, hipStream_t st);

@@ -206,6 +206,17 @@ SPARK_API int ds41_fp8_gemv_ex(const void* x, const void* w, const void* ws, flo
     if (m < 1 || m > 8 || n < 1 || k < 32 || k % 32 != 0 || (rpg && rpg % 32)) return 1;
     return launch_qgemv<1>(x, w, ws, y, m, n, k, xs, rpg, 0, st);
 }
+// reference ds41_mx.cu:1385-1393: the same product for up to 16 rows (there a tensor-core kernel whose cost does not grow with m);
+// here rows beyond 8 take a second pass of the same kernel, so a row's value does not depend on m
+SPARK_API int ds41_fp8_gemv_bx(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, int xs, int rpg, hipStream_t st)
+{
+    if (m < 1 || m > 16 || k % 64 || n % 8 || (rpg && rpg % 32)) return 1;
+    for (int r0 = 0; r0 < m; r0 += 8) {
+        const int rc = ds41_fp8_gemv_ex((const uint16_t*)x + (int64_t)r0 * xs, w, ws, y + (int64_t)r0 * n, m - r0 < 8 ? m - r0 : 8, n, k, xs, rpg, st);
+        if (rc) return rc;
+    }
+    return 0;
+}
 SPARK_API int ds41_fp8_gemv(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, hipStream_t st)
 {
     return ds41_fp8_gemv_ex(x, w, ws, y, m, n, k, k, 0, st);

@@ -38,6 +38,7 @@ SIGNATURES = {
     "ds41_mxfp4_gemv": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
     "ds41_fp8_gemv": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
     "ds41_fp8_gemv_ex": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
+    "ds41_fp8_gemv_bx": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
     "spark_fp8_block128_gemv": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
     "ds41_bf16_gemv": (i32, [vp, vp, vp, i32, i32, i32, vp]),
     # MXFP4 MoE

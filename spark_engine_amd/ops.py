@@ -166,6 +166,16 @@ def fp8_gemv(x, w, s):
     return y
 
 
+def fp8_gemv_bx(x, w, s, rpg=0):
+    """reference kern.rs fp8_gemv_bx (ds41_fp8_gemv_bx): up to 16 rows; rpg > 0 = block-diagonal groups of rpg weight rows."""
+    m = x.shape[0]
+    n = w.shape[0]
+    k = w.shape[1]
+    y = torch.empty(m, n, dtype=torch.float32, device=x.device)
+    _ck(_lib().ds41_fp8_gemv_bx(_p(_dev(x)), _p(_dev(w)), _p(_dev(s)), _p(y), m, n, k, x.stride(0), rpg, _st()), "ds41_fp8_gemv_bx")
+    return y
+
+
 def fp8_block128_gemv(x, w, scales, y=None):
     m, k = x.shape
     n = w.shape[0]

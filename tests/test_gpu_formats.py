@@ -164,6 +164,26 @@ def test_fp8_gemvs(ops, oracle, m):
     assert rel_l2(y, ref) < 1e-5
 
 
+def test_fp8_gemv_bx_up_to_16_rows_and_groups(ops, oracle):
+    g = synth.rng(150)
+    n, k, m = 256, 512, 13
+    w8, _ = synth.fp8_block_matrix(g, n, k)
+    s8 = g.integers(110, 128, (n // 32, k // 32), dtype=np.uint8)
+    x = synth.randn_bf16(g, (m, k))
+    y = host(ops.fp8_gemv_bx(dev_bf16(x), dev(w8), dev(s8)))
+    ref = oracle.fp8_e8m0_gemv(x, w8, s8)
+    assert rel_l2(y, ref) < 1e-5
+    y8 = host(ops.fp8_gemv(dev_bf16(x[:8]), dev(w8), dev(s8)))
+    assert np.array_equal(y[:8], y8)                                   # a row's value does not depend on the row count
+    # block-diagonal: weight rows [64 j, 64 j + 64) read input elements [j k, (j + 1) k) of their row
+    groups = n // 64
+    xg = synth.randn_bf16(g, (3, groups * k))
+    yg = host(ops.fp8_gemv_bx(dev_bf16(xg), dev(w8), dev(s8), rpg=64))
+    for j in range(groups):
+        refj = oracle.fp8_e8m0_gemv(np.ascontiguousarray(xg[:, j * k:(j + 1) * k]), w8, s8)[:, 64 * j:64 * j + 64]
+        assert rel_l2(yg[:, 64 * j:64 * j + 64], refj) < 1e-5
+
+
 def test_gemv_rejects_bad_shapes(ops):
     x = torch.zeros(9, 64, dtype=torch.bfloat16, device=DEV)
     w = torch.zeros(8, 32, dtype=torch.uint8, device=DEV)
