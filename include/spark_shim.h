@@ -39,6 +39,21 @@ SPARK_API int spark_exl3_fold(const void* trellis, const void* suh, const void* 
                               int64_t ldo, hipStream_t st);
 SPARK_API int qwen_exl3_fold(const void* trellis, const void* suh, const void* svh, int K, int N, int bits, void* out_f16, int64_t ldo,
                              hipStream_t st);
+/* Dense EXL3 linears for M <= 64 rows, trellis widths 3..6 bits, mul1 codebook: y = had128(had128(x * suh) @ inner) * svh in three
+ * steps or at once.  xh [M, K] fp16, part [S, M, N] fp32 (S = K slices, summed in order), cnt unused.  qwen_exl3_multi: up to 4
+ * linears on the same x (silu bit 0 with n = 2: y[0] = silu(linear 0) * linear 1); its mixed-input form (mg / mn) and side-stream
+ * fork (silu bit 2) are not provided (-5).  Replace engine-rs/shim/qwen_exl3.cu:70-206. */
+SPARK_API int qwen_exl3_had_in(const void* x, int x_f32, int64_t ldx, const void* suh, void* xh, int M, int K, hipStream_t st);
+SPARK_API int qwen_exl3_had_multi(const void* x, int64_t ldx, int M, int K, int n, const void* const* suh, void* const* xh, hipStream_t st);
+SPARK_API int qwen_exl3_gemv(const void* xh, const void* trellis, void* part, int M, int K, int N, int bits, int S, hipStream_t st);
+SPARK_API int qwen_exl3_finish(const void* part, int S, const void* svh, void* y, int y_f32, int64_t ldy, int M, int N, hipStream_t st);
+SPARK_API int qwen_exl3_finish_h(const void* part, const void* svh, void* y, int64_t ldy, int M, int N, hipStream_t st);
+SPARK_API int qwen_exl3_linear(const void* x, int64_t ldx, const void* suh, const void* trellis, const void* svh, void* part, void* y,
+                               int64_t ldy, void* cnt, int M, int K, int N, int bits, int S, hipStream_t st);
+SPARK_API int qwen_exl3_multi(const void* x, int64_t ldx, const void* mg, const void* mn, void* xout, int M, int K, int n,
+                              const void* const* suh, void* const* xh, const void* const* trellis, void* const* part, const int* N,
+                              const int* S, const void* const* svh, void* const* y, const int64_t* ldy, const int* bits, int silu,
+                              hipStream_t st);
 /* MXFP4: w [N, K/2] bytes (low nibble = even k), s [N, K/32] E8M0 -> fp32 [N, K].
  * Restates reference/ds41/kernel.py:122-131 (dequant_fp4_weight) and engine-rs/src/ds41/load.rs:338-349. */
 SPARK_API int spark_mxfp4_dequant(const void* w, const void* s, float* out, int N, int K, hipStream_t st);

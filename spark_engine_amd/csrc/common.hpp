@@ -28,7 +28,14 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f)
 }
 __device__ __forceinline__ float bf16_round(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { _Float16 v; __builtin_memcpy(&v, &h, 2); return (float)v; }
-__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { _Float16 v = (_Float16)f; uint16_t h; __builtin_memcpy(&h, &v, 2); return h; }   // RNE
+// binary32 -> fp16 bits, round to nearest even.  The argument is made opaque first: otherwise the compiler folds a multiply that
+// produced it into the conversion (one rounding of the exact product instead of the reference's two roundings: a different fp16
+// value when the binary32 product is a tie).
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f)
+{
+    asm volatile("" : "+v"(f));
+    _Float16 v = (_Float16)f; uint16_t h; __builtin_memcpy(&h, &v, 2); return h;
+}
 // E8M0 scale byte -> 2^(b-127) from the exponent bits (byte 0 gives 0.0)
 __device__ __forceinline__ float e8m0_to_f32(uint32_t b) { return __uint_as_float(b << 23); }
 // OCP E4M3 (fn) -> binary32.  Exponent and mantissa are dropped into binary32 and rescaled by 2^120, which also maps the

@@ -1,0 +1,249 @@
+// Dense EXL3 linears for a few rows (M <= 64), trellis widths 3..6 bits: y = had128(had128(x * suh) @ inner) * svh.
+//   reference engine-rs/shim/qwen_exl3.cu:66-206 (qwen_exl3_had_in / gemv / finish / finish_h / linear / had_multi / multi),
+//   kernels engine-rs/shim/qwen_exl3.cuh:165-183 (had_in), :292-413 (gemv), :560-629 (finish).
+// These are the projections next to the expert path (attention, shared expert); they are built for coverage of the shim's
+// ABI at any trellis width: one workgroup per (128 output columns, K slice) decodes a 16 x 128 strip of weights per k-tile into
+// LDS with the generic state extraction (the same code as the dequantisation surface, so the weights are the reference's bits)
+// and multiplies it with the transformed rows in binary32.  The partial sums of the K slices are added in slice order.
+#include "common.hpp"
+#include "exl3_decode.hpp"
+
+using namespace spk;
+
+namespace {
+
+constexpr int DM = 64;                 // most rows
+constexpr int DT = 256;                // threads
+
+// x [M, K] (fp32 or fp16, row stride ldx) -> xh [M, K] fp16 = had128(x * suh), one wave per (row, 128-block)
+template <bool XF32>
+__global__ __launch_bounds__(256) void had_in_kernel(const void* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ suh, uint16_t* __restrict__ xh,
+                                                     int M, int K)
+{
+    const int64_t wv = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63, nb = K / 128;
+    if (wv >= (int64_t)M * nb) return;
+    const int r = (int)(wv / nb), k = (int)(wv % nb) * 128 + 2 * lane;
+    float v0, v1;
+    if (XF32) { v0 = ((const float*)x)[r * ldx + k]; v1 = ((const float*)x)[r * ldx + k + 1]; }
+    else { v0 = f16_bits_to_f32(((const uint16_t*)x)[r * ldx + k]); v1 = f16_bits_to_f32(((const uint16_t*)x)[r * ldx + k + 1]); }
+    v0 *= f16_bits_to_f32(suh[k]); v1 *= f16_bits_to_f32(suh[k + 1]);
+    fwht128(v0, v1, lane);
+    *(uint32_t*)(xh + (int64_t)r * K + k) = (uint32_t)f32_to_f16_bits(v0) | ((uint32_t)f32_to_f16_bits(v1) << 16);
+}
+
+// part[s][m][n] = xh[m, slice s of K] @ inner[slice, n]; grid (N / 128, S).  XMODE 0: xh fp16 given; 1: x fp32 + suh, transformed here.
+template <int CBK, int XMODE>
+__global__ __launch_bounds__(DT) void dense_gemv_kernel(const void* __restrict__ xin, int64_t ldx, const uint16_t* __restrict__ suh,
+                                                        const uint32_t* __restrict__ tr, float* __restrict__ part, int M, int K, int N, int bits, int kts, int kpad)
+{
+    extern __shared__ __align__(16) unsigned char sm[];
+    const int Kt = K / 16, Nt = N / 16, nw = 8 * bits;
+    const int nb = blockIdx.x, s = blockIdx.y;
+    const int kt0 = s * kts, kt1 = min(Kt, kt0 + kts), nkt = max(0, kt1 - kt0);
+    uint16_t* xs = (uint16_t*)sm;                                          // [M][kpad] fp16 of the transformed rows from k0 on: the slice widened to whole Hadamard blocks
+    uint16_t* wl = xs + (size_t)M * kpad;                                  // [16][128] decoded strip
+    uint32_t* tw = (uint32_t*)(wl + 16 * 128);                             // [8][48] words of the 8 tiles
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int k0 = kt0 * 16 / 128 * 128;                                   // first Hadamard block touching the slice
+    const int off = kt0 * 16 - k0;
+    if (XMODE == 0) {
+        for (int i = tid; i < M * (kpad / 2); i += DT) {
+            const int r = i / (kpad / 2), c = (i % (kpad / 2)) * 2;
+            *(uint32_t*)(xs + (size_t)r * kpad + c) = k0 + c < K ? *(const uint32_t*)((const uint16_t*)xin + (int64_t)r * K + k0 + c) : 0u;
+        }
+    } else {
+        const int nblk = kpad / 128;
+        for (int u = wave; u < M * nblk; u += DT / 64) {
+            const int r = u / nblk, k = k0 + (u % nblk) * 128 + 2 * lane;
+            float v0 = 0.f, v1 = 0.f;
+            if (k < K) {
+                v0 = ((const float*)xin)[r * ldx + k] * f16_bits_to_f32(suh[k]);
+                v1 = ((const float*)xin)[r * ldx + k + 1] * f16_bits_to_f32(suh[k + 1]);
+            }
+            fwht128(v0, v1, lane);
+            *(uint32_t*)(xs + (size_t)r * kpad + (k - k0)) = (uint32_t)f32_to_f16_bits(v0) | ((uint32_t)f32_to_f16_bits(v1) << 16);
+        }
+    }
+    // thread -> output column tid % 128 for the rows of its half (even / odd rows)
+    const int col = tid & 127, half = tid >> 7;
+    float acc[DM / 2];
+#pragma unroll
+    for (int i = 0; i < DM / 2; ++i) acc[i] = 0.f;
+    for (int kt = 0; kt < nkt; ++kt) {
+        __syncthreads();
+        for (int i = tid; i < 8 * nw; i += DT) {
+            const int t = i / nw, j = i % nw;
+            tw[t * 48 + j] = tr[((int64_t)(kt0 + kt) * Nt + nb * 8 + t) * nw + j];
+        }
+        __syncthreads();
+        for (int i = tid; i < 8 * 256; i += DT) {                          // one weight per thread-step: tile i / 256, position i % 256
+            const int t = i >> 8, p = i & 255;
+            int row, c;
+            tile_pos(p, row, c);
+            const _Float16 v = cb_decode<CBK>(tile_state(tw + t * 48, bits, p));
+            uint16_t hb; __builtin_memcpy(&hb, &v, 2);
+            wl[row * 128 + t * 16 + c] = hb;
+        }
+        __syncthreads();
+        float wv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) wv[r] = f16_bits_to_f32(wl[r * 128 + col]);
+        const uint16_t* xk = xs + off + kt * 16;
+#pragma unroll
+        for (int i = 0; i < DM / 2; ++i) {
+            const int m = 2 * i + half;
+            if (m < M) {
+                const uint16_t* xr = xk + (size_t)m * kpad;
+                float a = acc[i];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) a = __builtin_fmaf(f16_bits_to_f32(xr[r]), wv[r], a);
+                acc[i] = a;
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < DM / 2; ++i) {
+        const int m = 2 * i + half;
+        if (m < M) part[((int64_t)s * M + m) * N + nb * 128 + col] = acc[i];
+    }
+}
+
+// y[m, n] = had128(sum_s part[s][m][:]) * svh (the silu form: y = silu(linear 0) * linear 1); one wave per (row, 128-block)
+template <bool PH, bool YF32>
+__global__ __launch_bounds__(256) void finish_kernel(const void* __restrict__ part, int S, const uint16_t* __restrict__ svh, void* __restrict__ y, int64_t ldy,
+                                                     int M, int N, const float* __restrict__ part2, const uint16_t* __restrict__ svh2)
+{
+    const int64_t wv = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63, nb = N / 128;
+    if (wv >= (int64_t)M * nb) return;
+    const int r = (int)(wv / nb), n = (int)(wv % nb) * 128 + 2 * lane;
+    auto one = [&](const void* p, const uint16_t* sv, float& o0, float& o1) {
+        float v0 = 0.f, v1 = 0.f;
+        for (int s = 0; s < S; ++s) {
+            if (PH) { v0 += f16_bits_to_f32(((const uint16_t*)p)[((int64_t)s * M + r) * N + n]); v1 += f16_bits_to_f32(((const uint16_t*)p)[((int64_t)s * M + r) * N + n + 1]); }
+            else { v0 += ((const float*)p)[((int64_t)s * M + r) * N + n]; v1 += ((const float*)p)[((int64_t)s * M + r) * N + n + 1]; }
+        }
+        fwht128(v0, v1, lane);
+        o0 = v0 * f16_bits_to_f32(sv[n]); o1 = v1 * f16_bits_to_f32(sv[n + 1]);
+    };
+    float a0, a1;
+    one(part, svh, a0, a1);
+    if (part2) {
+        float b0, b1;
+        one(part2, svh2, b0, b1);
+        a0 = a0 / (1.0f + __expf(-a0)) * b0; a1 = a1 / (1.0f + __expf(-a1)) * b1;
+    }
+    if (YF32) { ((float*)y)[r * ldy + n] = a0; ((float*)y)[r * ldy + n + 1] = a1; }
+    else { ((uint16_t*)y)[r * ldy + n] = f32_to_f16_bits(a0); ((uint16_t*)y)[r * ldy + n + 1] = f32_to_f16_bits(a1); }
+}
+
+int launch_gemv(int xmode, const void* x, int64_t ldx, const void* suh, const void* trellis, void* part, int M, int K, int N, int bits, int S, int codebook,
+                hipStream_t st)
+{
+    if (M < 1 || M > DM || K < 128 || N < 128 || K % 128 || N % 128 || S < 1) return -1;
+    if (bits < 3 || bits > 6) return -2;
+    const int kts = (K / 16 + S - 1) / S;
+    const int kpad = (kts * 16 + 127) / 128 * 128 + 128;                 // a slice may start inside a Hadamard block
+    const size_t smem = (size_t)M * kpad * 2 + 16 * 128 * 2 + 8 * 48 * 4;
+    if (smem > 160 * 1024) return -1;
+    const dim3 grid(N / 128, S);
+#define DG(CB, XM)                                                                                                                              \
+    do {                                                                                                                                        \
+        static bool attr = hipFuncSetAttribute((const void*)dense_gemv_kernel<CB, XM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess; \
+        if (!attr) return -3;                                                                                                                   \
+        dense_gemv_kernel<CB, XM><<<grid, DT, smem, st>>>(x, ldx, (const uint16_t*)suh, (const uint32_t*)trellis, (float*)part, M, K, N, bits, kts, kpad); \
+    } while (0)
+    if (codebook == CB_MCG) { if (xmode) DG(CB_MCG, 1); else DG(CB_MCG, 0); }
+    else { if (xmode) DG(CB_MUL1, 1); else DG(CB_MUL1, 0); }
+#undef DG
+    return launch_status();
+}
+
+}  // namespace
+
+// ================================================================ C ABI (reference engine-rs/shim/qwen_exl3.cu)
+
+// x [M, K] (fp32 if x_f32 else fp16, row stride ldx) -> xh [M, K] fp16.  reference qwen_exl3.cu:137-147
+SPARK_API int qwen_exl3_had_in(const void* x, int x_f32, int64_t ldx, const void* suh, void* xh, int M, int K, hipStream_t st)
+{
+    if (M < 1 || K < 128 || K % 128) return -1;
+    const int64_t waves = (int64_t)M * (K / 128);
+    const unsigned blocks = (unsigned)((waves * 64 + 255) / 256);
+    if (x_f32) had_in_kernel<true><<<blocks, 256, 0, st>>>(x, ldx, (const uint16_t*)suh, (uint16_t*)xh, M, K);
+    else had_in_kernel<false><<<blocks, 256, 0, st>>>(x, ldx, (const uint16_t*)suh, (uint16_t*)xh, M, K);
+    return launch_status();
+}
+// had_in of up to 4 linears from the same x fp32.  reference qwen_exl3.cu:70-80
+SPARK_API int qwen_exl3_had_multi(const void* x, int64_t ldx, int M, int K, int n, const void* const* suh, void* const* xh, hipStream_t st)
+{
+    if (n < 1 || n > 4 || K % 128) return -1;
+    for (int i = 0; i < n; ++i) {
+        const int rc = qwen_exl3_had_in(x, 1, ldx, suh[i], xh[i], M, K, st);
+        if (rc) return rc;
+    }
+    return 0;
+}
+// xh [M <= 64, K] fp16, trellis [K/16, N/16, 16*bits] int16 -> part [S, M, N] fp32 (mul1 codebook).  reference qwen_exl3.cu:171-184
+SPARK_API int qwen_exl3_gemv(const void* xh, const void* trellis, void* part, int M, int K, int N, int bits, int S, hipStream_t st)
+{
+    return launch_gemv(0, xh, K, nullptr, trellis, part, M, K, N, bits, S, CB_MUL1, st);
+}
+// part [S, M, N] fp32 -> y [M, N] (fp32 if y_f32 else fp16, row stride ldy).  reference qwen_exl3.cu:187-197
+SPARK_API int qwen_exl3_finish(const void* part, int S, const void* svh, void* y, int y_f32, int64_t ldy, int M, int N, hipStream_t st)
+{
+    if (M < 1 || N < 128 || N % 128 || S < 1) return -1;
+    const unsigned blocks = (unsigned)(((int64_t)M * (N / 128) * 64 + 255) / 256);
+    if (y_f32) finish_kernel<false, true><<<blocks, 256, 0, st>>>(part, S, (const uint16_t*)svh, y, ldy, M, N, nullptr, nullptr);
+    else finish_kernel<false, false><<<blocks, 256, 0, st>>>(part, S, (const uint16_t*)svh, y, ldy, M, N, nullptr, nullptr);
+    return launch_status();
+}
+// part [M, N] fp16 (one slice) -> y [M, N] fp32.  reference qwen_exl3.cu:199-206
+SPARK_API int qwen_exl3_finish_h(const void* part, const void* svh, void* y, int64_t ldy, int M, int N, hipStream_t st)
+{
+    if (M < 1 || N < 128 || N % 128) return -1;
+    const unsigned blocks = (unsigned)(((int64_t)M * (N / 128) * 64 + 255) / 256);
+    finish_kernel<true, true><<<blocks, 256, 0, st>>>(part, 1, (const uint16_t*)svh, y, ldy, M, N, nullptr, nullptr);
+    return launch_status();
+}
+// x [M <= 64, K] fp32 -> y [M, N] fp32; part: scratch [S, M, N] fp32; cnt is not used here (two launches, no counters).
+// reference qwen_exl3.cu:150-168
+SPARK_API int qwen_exl3_linear(const void* x, int64_t ldx, const void* suh, const void* trellis, const void* svh, void* part, void* y, int64_t ldy, void* cnt,
+                               int M, int K, int N, int bits, int S, hipStream_t st)
+{
+    (void)cnt;
+    const int rc = launch_gemv(1, x, ldx, suh, trellis, part, M, K, N, bits, S, CB_MUL1, st);
+    if (rc) return rc;
+    return qwen_exl3_finish(part, S, svh, y, 1, ldy, M, N, st);
+}
+// Up to 4 linears on the same x fp32 [M <= 64, K]; silu bit 0 (n = 2): y[0] = silu(linear 0) * linear 1.  The mixed-input form
+// (mg / mn non-null) and the side-stream fork (silu bit 2) belong to the model graph and are not provided: -5.
+// reference qwen_exl3.cu:89-134
+SPARK_API int qwen_exl3_multi(const void* x, int64_t ldx, const void* mg, const void* mn, void* xout, int M, int K, int n, const void* const* suh,
+                              void* const* xh, const void* const* trellis, void* const* part, const int* N, const int* S, const void* const* svh, void* const* y,
+                              const int64_t* ldy, const int* bits, int silu, hipStream_t st)
+{
+    (void)xout; (void)xh;
+    if (n < 1 || n > 4 || M > 64 || K % 128) return -1;
+    if (mg || mn || (silu & 4)) return -5;
+    for (int i = 0; i < n; ++i) {
+        if (N[i] % 128) return -1;
+        if (bits[i] < 3 || bits[i] > 6) return -2;
+    }
+    for (int i = 0; i < n; ++i) {
+        const int rc = launch_gemv(1, x, ldx, suh[i], trellis[i], part[i], M, K, N[i], bits[i], S[i], CB_MUL1, st);
+        if (rc) return rc;
+    }
+    if (silu & 1) {
+        if (n != 2 || N[0] != N[1] || S[0] != S[1]) return -3;
+        const unsigned blocks = (unsigned)(((int64_t)M * (N[0] / 128) * 64 + 255) / 256);
+        finish_kernel<false, true><<<blocks, 256, 0, st>>>(part[0], S[0], (const uint16_t*)svh[0], y[0], ldy[0], M, N[0], (const float*)part[1],
+                                                           (const uint16_t*)svh[1]);
+        return launch_status();
+    }
+    for (int i = 0; i < n; ++i) {
+        const int rc = qwen_exl3_finish(part[i], S[i], svh[i], y[i], 1, ldy[i], M, N[i], st);
+        if (rc) return rc;
+    }
+    return 0;
+}

@@ -17,6 +17,13 @@ SIGNATURES = {
     "qwen_exl3_reconstruct": (i32, [vp, vp, i32, i32, i32, vp]),
     "spark_exl3_fold": (i32, [vp, vp, vp, i32, i32, i32, i32, vp, i64, vp]),
     "qwen_exl3_fold": (i32, [vp, vp, vp, i32, i32, i32, vp, i64, vp]),
+    "qwen_exl3_had_in": (i32, [vp, i32, i64, vp, vp, i32, i32, vp]),
+    "qwen_exl3_had_multi": (i32, [vp, i64, i32, i32, i32, vp, vp, vp]),
+    "qwen_exl3_gemv": (i32, [vp, vp, vp, i32, i32, i32, i32, i32, vp]),
+    "qwen_exl3_finish": (i32, [vp, i32, vp, vp, i32, i64, i32, i32, vp]),
+    "qwen_exl3_finish_h": (i32, [vp, vp, vp, i64, i32, i32, vp]),
+    "qwen_exl3_linear": (i32, [vp, i64, vp, vp, vp, vp, vp, i64, vp, i32, i32, i32, i32, i32, vp]),
+    "qwen_exl3_multi": (i32, [vp, i64, vp, vp, vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp]),
     "spark_mxfp4_dequant": (i32, [vp, vp, vp, i32, i32, vp]),
     "spark_fp8_block_dequant": (i32, [vp, vp, vp, i32, i32, i32, vp]),
     "spark_fp8_e8m0_dequant": (i32, [vp, vp, vp, i32, i32, vp]),

@@ -54,6 +54,60 @@ def exl3_fold(trellis, suh, svh, codebook=2):
     return out
 
 
+# ---------------------------------------------------------------- dense EXL3 linears (reference qwen/ffi.rs exl3_* wrappers)
+
+def exl3_had_in(x, suh):
+    """x f32 | f16 [M, K] -> xh f16 [M, K] = had128(x * suh)."""
+    M, K = x.shape
+    xh = torch.empty(M, K, dtype=torch.float16, device=x.device)
+    _ck(_lib().qwen_exl3_had_in(_p(x), int(x.dtype == torch.float32), x.stride(0), _p(_dev(suh)), _p(xh), M, K, _st()), "qwen_exl3_had_in")
+    return xh
+
+
+def exl3_gemv(xh, trellis, S=4):
+    """xh f16 [M, K], trellis int16 [K/16, N/16, 16*bits] -> part f32 [S, M, N]."""
+    M, K = xh.shape
+    Kt, Nt, W = trellis.shape
+    part = torch.empty(S, M, Nt * 16, dtype=torch.float32, device=xh.device)
+    _ck(_lib().qwen_exl3_gemv(_p(_dev(xh)), _p(_dev(trellis)), _p(part), M, K, Nt * 16, W // 16, S, _st()), "qwen_exl3_gemv")
+    return part
+
+
+def exl3_finish(part, svh, f32=True):
+    S, M, N = part.shape
+    y = torch.empty(M, N, dtype=torch.float32 if f32 else torch.float16, device=part.device)
+    _ck(_lib().qwen_exl3_finish(_p(_dev(part)), S, _p(_dev(svh)), _p(y), int(f32), N, M, N, _st()), "qwen_exl3_finish")
+    return y
+
+
+def exl3_linear(x, suh, trellis, svh, S=4):
+    """x f32 [M, K] -> y f32 [M, N] (had_in + gemv + finish)."""
+    M, K = x.shape
+    Kt, Nt, W = trellis.shape
+    N = Nt * 16
+    part = torch.empty(S, M, N, dtype=torch.float32, device=x.device)
+    y = torch.empty(M, N, dtype=torch.float32, device=x.device)
+    _ck(_lib().qwen_exl3_linear(_p(x), x.stride(0), _p(_dev(suh)), _p(_dev(trellis)), _p(_dev(svh)), _p(part), _p(y), N, None, M, K, N, W // 16, S, _st()),
+        "qwen_exl3_linear")
+    return y
+
+
+def exl3_multi(x, linears, S=4, silu=False):
+    """x f32 [M, K]; linears = [(suh, trellis, svh), ...] (at most 4) -> list of y f32 [M, N_i] (one tensor with silu)."""
+    M, K = x.shape
+    n = len(linears)
+    Ns = [lin[1].shape[1] * 16 for lin in linears]
+    bits = [lin[1].shape[2] // 16 for lin in linears]
+    parts = [torch.empty(S, M, N, dtype=torch.float32, device=x.device) for N in Ns]
+    ys = [torch.empty(M, N, dtype=torch.float32, device=x.device) for N in Ns]
+    vpa = lambda ts: (C.c_void_p * n)(*[t.data_ptr() for t in ts])
+    ia = lambda vs: (C.c_int * n)(*vs)
+    _ck(_lib().qwen_exl3_multi(_p(x), x.stride(0), None, None, None, M, K, n, vpa([lin[0] for lin in linears]), None, vpa([lin[1] for lin in linears]),
+                               vpa(parts), ia(Ns), ia([S] * n), vpa([lin[2] for lin in linears]), vpa(ys), (C.c_int64 * n)(*Ns), ia(bits), int(silu), _st()),
+        "qwen_exl3_multi")
+    return ys[0] if silu else ys
+
+
 def mxfp4_dequant(w, s):
     N, K = w.shape[0], w.shape[1] * 2
     out = torch.empty(N, K, dtype=torch.float32, device=w.device)

@@ -1,0 +1,81 @@
+"""GPU parity of the dense EXL3 linears (the reference shim's qwen_exl3_had_in / gemv / finish / linear / multi) against the
+CPU oracle, trellis widths 3..6 bits.  had_in is bit-exact; the products are held to rel-L2 <= 1e-3 (measured ~1e-6: the
+weights are bit-exact, the sums differ in order)."""
+import numpy as np
+import pytest
+import torch
+
+from spark_engine_amd import synth
+from tests.gpu_util import DEV, dev, dev_f16, host, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from spark_engine_amd import ops
+    return ops
+
+
+def _f16(bits):
+    return np.asarray(bits, np.uint16).view(np.float16).astype(np.float32)
+
+
+def _reference(oracle, x, tr, suh, svh):
+    """y = had128(had128(x * suh) rounded to fp16 @ inner) * svh, sums in float64"""
+    M, K = x.shape
+    N = tr.shape[1] * 16
+    xh = np.stack([_f16(oracle.had_in(x[m], suh)) for m in range(M)])
+    inner = _f16(oracle.decode_inner(tr, 2))
+    t = (xh.astype(np.float64) @ inner.astype(np.float64)).astype(np.float32)
+    y = np.empty((M, N), np.float32)
+    for m in range(M):
+        for b in range(N // 128):
+            y[m, b * 128:(b + 1) * 128] = oracle.fwht128(t[m, b * 128:(b + 1) * 128])
+    return y * _f16(svh)[None, :], xh
+
+
+@pytest.mark.parametrize("bits", [3, 4, 5, 6])
+def test_linear_steps_and_fused_form(ops, oracle, bits):
+    g = synth.rng(500 + bits)
+    M, K, N, S = 5, 512, 384, 3                                         # S = 3: slices that start inside a Hadamard block
+    tr, suh, svh = synth.exl3_matrix(g, K, N, bits)
+    x = g.standard_normal((M, K)).astype(np.float32)
+    ref, xh_ref = _reference(oracle, x, tr, suh, svh)
+    xh = ops.exl3_had_in(dev(x), dev_f16(suh))
+    assert np.array_equal(host(xh).view(np.float16).astype(np.float32), xh_ref)       # bit-exact transform
+    part = ops.exl3_gemv(xh, dev(tr), S=S)
+    y = host(ops.exl3_finish(part, dev_f16(svh)))
+    assert rel_l2(y, ref) <= 1e-3, rel_l2(y, ref)
+    y2 = host(ops.exl3_linear(dev(x), dev_f16(suh), dev(tr), dev_f16(svh), S=S))
+    assert np.array_equal(y, y2)                                         # the one-call form does the same arithmetic
+    yh = host(ops.exl3_finish(part, dev_f16(svh), f32=False)).view(np.float16).astype(np.float32)
+    assert np.array_equal(yh, y.astype(np.float16).astype(np.float32))
+    x16 = x.astype(np.float16)
+    xh16 = ops.exl3_had_in(dev_f16(x16.view(np.uint16)), dev_f16(suh))  # fp16 input form
+    _, xh_ref16 = _reference(oracle, x16.astype(np.float32), tr, suh, svh)
+    assert np.array_equal(host(xh16).view(np.float16).astype(np.float32), xh_ref16)
+
+
+def test_multi_and_silu(ops, oracle):
+    g = synth.rng(510)
+    M, K = 3, 256
+    lins = [synth.exl3_matrix(g, K, N, b) for N, b in ((256, 4), (256, 5), (128, 6))]
+    x = g.standard_normal((M, K)).astype(np.float32)
+    dl = [(dev_f16(s), dev(t), dev_f16(v)) for t, s, v in lins]
+    ys = ops.exl3_multi(dev(x), dl, S=2)
+    refs = [_reference(oracle, x, t, s, v)[0] for t, s, v in lins]
+    for y, ref in zip(ys, refs):
+        assert rel_l2(host(y), ref) <= 1e-3
+    ysilu = host(ops.exl3_multi(dev(x), dl[:2], S=2, silu=True))
+    a, b = refs[0].astype(np.float64), refs[1].astype(np.float64)
+    assert rel_l2(ysilu, a / (1 + np.exp(-a)) * b) <= 1e-3
+
+
+def test_dense_rejects_bad_arguments(ops):
+    x = torch.zeros(2, 200, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.exl3_had_in(x, torch.zeros(200, dtype=torch.float16, device=DEV))         # K % 128 != 0 -> -1
+    xh = torch.zeros(2, 256, dtype=torch.float16, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.exl3_gemv(xh, torch.zeros(16, 8, 16 * 7, dtype=torch.int16, device=DEV))  # 7-bit trellis -> -2
