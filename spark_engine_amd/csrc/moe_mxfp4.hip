@@ -327,7 +327,7 @@ int moe_launch(const uint8_t* xq, const uint8_t* xs, int R, const int64_t* idx, 
     uint8_t* hs = (uint8_t*)(base + l.hs);
     float* out = (float*)(base + l.out);
     group_kernel<<<1, 1024, 0, st>>>(idx, rw, R, topk, n_shared, E, GR, G, items, pairmap, prow, pw, G + 4, 64);
-    const WMat m1{w1, s1, I, H}, m3{w3, s3, I, H}, m2{w2, s2, H, I};
+    const WMat m1{w1, s1, I, H, (int64_t)ET * I / 8}, m3{w3, s3, I, H, (int64_t)ET * I / 8}, m2{w2, s2, H, I, (int64_t)ET * H / 8};
     up_kernel<LAYOUT><<<dim3(I / 32, Gm), 64 * UP_WAVES, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
     down_kernel<LAYOUT><<<dim3(H / 32, Gm), 64 * DN_WAVES, 0, st>>>(hq, hs, m2, H, I, G, items, out);
     if (!skip_combine) {
@@ -450,7 +450,9 @@ SPARK_API int ds41_moe_mx_ex(const void* xq, const void* xs, int R, const int64_
                              hipStream_t st)
 {
     if (R < 1 || I % 128 != 0 || E > 384 || topk < 1) return 1;
-    if (g_s2) return 5;                                        // 2-bit coded scale blobs are not decoded here
+    if (g_s2)                                                  // s1 / s3 / s2 are 2-bit coded scale blobs
+        return moe_launch<L_MX8S2>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3,
+                                   (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, DS41_H, I, topk, E, 0, add, y, ws, skip_combine, st);
     return moe_launch<L_MX8>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3, (const uint8_t*)s3,
                              (const uint8_t*)w2, (const uint8_t*)s2, DS41_H, I, topk, E, 0, add, y, ws, skip_combine, st);
 }

@@ -12,12 +12,17 @@ namespace mx {
 
 constexpr int REC = 4352;              // bytes per T16 record
 
-enum Layout { L_T16 = 0, L_NATURAL = 1, L_PACK8 = 2, L_MX8 = 3 };
+// L_MX8S2: the codes of L_MX8 with the scales in the reference's lossless 2-bit coding (engine-rs/shim/ds41_mx.cu:64-91,
+// engine-rs/src/ds41/kern.rs:747-770): one blob per matrix of T = experts * rows / 8 tiles and S = K / 128 steps =
+// desc [T][16] (bytes 0-7 the rows' base scales, bytes 8-11 an int32 index into raw or -1), codes [T][S][8 rows] (four 2-bit
+// offsets per byte, block b in bits 2b..2b+1), raw [n_raw][S][8][4] (tiles with a row whose scales span more than 3).
+enum Layout { L_T16 = 0, L_NATURAL = 1, L_PACK8 = 2, L_MX8 = 3, L_MX8S2 = 4 };
 
 struct WMat {                          // one stacked weight matrix [E, rows, K]
     const uint8_t* w;
     const uint8_t* s;
     int rows, K;                       // per expert
+    int64_t tiles8;                    // experts * rows / 8 (locates the sections of a 2-bit coded scale blob)
 };
 
 // ---- A operand: the 4 steps of K group kg of the 16 rows starting at row0 (row0 % 16 == 0) of expert e
@@ -49,11 +54,20 @@ __device__ __forceinline__ void load_group(const WMat& m, int e, int row0, int k
                 const uint4 v = ld_stream16(m.w + (t8 * steps + step) * 512 + (row & 7) * 64 + g * 16);
                 c[s] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
                 sb = m.s[(t8 * steps + step) * 32 + (row & 7) * 4 + g];
-            } else {                                        // L_MX8: [rows/8][K/128][8][4 q][4 b][4]
+            } else {                                        // L_MX8 / L_MX8S2: [rows/8][K/128][8][4 q][4 b][4]
                 const int64_t t8 = row >> 3;
-                const uint32_t* p = (const uint32_t*)(m.w + (t8 * steps + step) * 512 + (row & 7) * 64 + g * 4);
+                const int r8 = (int)(row & 7);
+                const uint32_t* p = (const uint32_t*)(m.w + (t8 * steps + step) * 512 + r8 * 64 + g * 4);
                 c[s] = v4i{(int)p[0], (int)p[4], (int)p[8], (int)p[12]};
-                sb = m.s[(t8 * steps + step) * 32 + (row & 7) * 4 + g];
+                if constexpr (LAYOUT == L_MX8) sb = m.s[(t8 * steps + step) * 32 + r8 * 4 + g];
+                else {
+                    const uint32_t* d = (const uint32_t*)(m.s + t8 * 16);
+                    const uint8_t* code = m.s + m.tiles8 * 16;
+                    const uint8_t* raw = code + m.tiles8 * steps * 8;
+                    const int ri = (int)d[2];
+                    if (ri >= 0) sb = raw[((int64_t)ri * steps + step) * 32 + r8 * 4 + g];
+                    else sb = ((d[r8 >> 2] >> (8 * (r8 & 3))) & 0xffu) + ((code[(t8 * steps + step) * 8 + r8] >> (2 * g)) & 3u);
+                }
             }
             sc4 = (sc4 & ~(0xffu << (8 * s))) | (sb << (8 * s));
         }

@@ -494,8 +494,9 @@ int mx_fused_launch(const void* x, const void* xs, int R, const int64_t* idx, co
     char* b = (char*)ws;
     MArgs a;
     a.x = x; a.xs = (const uint8_t*)xs; a.idx = idx; a.rw = rw;
-    a.w1 = WMat{(const uint8_t*)w1, (const uint8_t*)s1, I, H}; a.w3 = WMat{(const uint8_t*)w3, (const uint8_t*)s3, I, H};
-    a.w2 = WMat{(const uint8_t*)w2, (const uint8_t*)s2, H, I};
+    const int64_t ET = E + n_shared;
+    a.w1 = WMat{(const uint8_t*)w1, (const uint8_t*)s1, I, H, ET * I / 8}; a.w3 = WMat{(const uint8_t*)w3, (const uint8_t*)s3, I, H, ET * I / 8};
+    a.w2 = WMat{(const uint8_t*)w2, (const uint8_t*)s2, H, I, ET * H / 8};
     a.add = add; a.y = y;
     a.hc = (uint32_t*)(b + p.hc); a.hsw = (uint32_t*)(b + p.hsw); a.yd = (float*)(b + p.yd); a.err = (int*)b;
     a.R = R; a.TT = p.TT; a.topk = topk; a.E = E; a.P = p.P; a.Gmax = p.Gmax; a.H = H; a.I = I; a.NJ = p.NJ; a.NBD = p.NBD; a.nU = p.nU;

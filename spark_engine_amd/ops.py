@@ -342,6 +342,31 @@ def moe_pack_mx(wp):
     return wp.view(e * rows // 8, steps, 8, 4, 4, 4).permute(0, 1, 2, 4, 3, 5).contiguous().view(e, rows, kb)
 
 
+def moe_scales_s2(sp):
+    """reference kern.rs moe_scales_s2: tile-packed scales [E, rows, K/32] (moe_pack) -> the lossless 2-bit coded blob
+    (desc [tiles][16] | codes [tiles][steps][8] | raw words of the tiles with a row spanning more than 3), uint8.
+    Returns (blob, raw tiles, tiles)."""
+    e, rows, nb = sp.shape
+    tiles, steps = e * rows // 8, nb // 4
+    v = sp.view(tiles, steps, 8, 4).to(torch.int16)
+    mn = v.amin(dim=(1, 3))                                             # [tiles, 8]
+    raw = ((v.amax(dim=(1, 3)) - mn) > 3).any(dim=1)                    # [tiles]
+    code = (v - mn.view(tiles, 1, 8, 1)).clamp(0, 3)
+    wts = torch.tensor([1, 4, 16, 64], dtype=torch.int16, device=sp.device).view(1, 1, 1, 4)
+    cb = (code * wts).sum(dim=3).to(torch.uint8).contiguous()           # [tiles, steps, 8]
+    ri = raw.to(torch.int32).cumsum(0).to(torch.int32) - 1
+    ri = torch.where(raw, ri, torch.full_like(ri, -1)).contiguous()
+    rawt = sp.view(tiles, steps * 32)[raw]
+    desc = torch.cat([mn.to(torch.uint8), ri.view(torch.uint8).view(tiles, 4), torch.zeros(tiles, 4, dtype=torch.uint8, device=sp.device)], dim=1)
+    blob = torch.cat([desc.reshape(-1), cb.reshape(-1), rawt.contiguous().reshape(-1)])
+    return blob.contiguous(), int(raw.sum().item()), tiles
+
+
+def moe_s2_set(on):
+    """reference kern.rs moe_s2_set: the scale tensors handed to ds41_moe_mx* are 2-bit coded blobs."""
+    _lib().ds41_moe_mx_set_s2(int(bool(on)))
+
+
 def ds41_moe_mx(xq, xs, idx, rw, w, I, add=None, skip_combine=False, ws=None):
     """reference kern.rs moe_mx_par / ds41_moe_mx_ex: hidden 5120, weights w = (w1, s1, w3, s3, w2, s2) in the mx tile layout."""
     R = xq.shape[0]

@@ -124,3 +124,32 @@ def test_ds41_reference_symbols_tile_layouts(ops, oracle):
         assert L.ds41_moe_mx_combine_rows(C.c_void_p(wsb3.data_ptr()), R, I, topk, E, C.c_void_p(add_d.data_ptr()), C.c_void_p(y4.data_ptr()), r0, 1, st) == 0
     torch.cuda.synchronize()
     assert np.array_equal(host(y4), host(y))
+
+
+def test_ds41_two_bit_coded_scales(ops, oracle):
+    # the reference's lossless 2-bit scale coding (kern.rs moe_scales_s2): nearly constant scales are coded, a tile with a wide
+    # row keeps its raw words; the kernels must see the same scale bytes either way
+    g = synth.rng(214)
+    R, H, I, E, topk = 3, 5120, 128, 4, 2
+    ws, x, idx, rw = _case(g, R, H, I, E, topk, 0, smin=119)
+    ws = [a.copy() for a in ws]
+    for s in (ws[1], ws[3], ws[5]):
+        s[:] = g.integers(120, 123, s.shape, dtype=np.uint8)           # span <= 3 everywhere: coded tiles
+    ws[1][1, 9, 5] = 110                                                # one wide row: its tile stays raw
+    ws[5][2, 700, 1] = 127
+    ref = oracle.mxfp4_moe(x, idx, rw, *ws)
+    d = [dev(a) for a in ws]
+    p1, ps1 = ops.moe_pack(d[0], d[1]); p3, ps3 = ops.moe_pack(d[2], d[3]); p2, ps2 = ops.moe_pack(d[4], d[5])
+    xq, xs = ops.act_quant_fp8(dev_bf16(x))
+    packed = (ops.moe_pack_mx(p1), ops.moe_pack_mx(p3), ops.moe_pack_mx(p2))
+    y_raw, _ = ops.ds41_moe_mx(xq, xs, dev(idx), dev(rw), (packed[0], ps1, packed[1], ps3, packed[2], ps2), I)
+    b1, n1, t1 = ops.moe_scales_s2(ps1); b3, n3, _ = ops.moe_scales_s2(ps3); b2, n2, t2 = ops.moe_scales_s2(ps2)
+    assert (n1, n3, n2) == (1, 0, 1) and t1 == E * I // 8 and t2 == E * H // 8
+    assert b3.numel() == t1 * 16 + t1 * (H // 128) * 8                  # a quarter of the raw bytes + 16 per tile
+    ops.moe_s2_set(True)
+    try:
+        y_s2, _ = ops.ds41_moe_mx(xq, xs, dev(idx), dev(rw), (packed[0], b1, packed[1], b3, packed[2], b2), I)
+    finally:
+        ops.moe_s2_set(False)
+    assert np.array_equal(host(y_s2), host(y_raw))
+    assert rel_l2(host(y_s2), ref) <= TOL
