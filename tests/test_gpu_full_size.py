@@ -1,0 +1,87 @@
+"""The benchmark configurations at their full shapes.  Where the CPU oracle would take minutes (2048 tokens through 384
+experts) the check goes through properties that do not depend on size: a token row of the prefill-sized call must equal,
+bit for bit, the same row sent alone through the decode path (the kernels promise batch-size independence), and a sample
+of rows is held against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from spark_engine_amd import synth
+from tests.gpu_util import DEV, dev, dev_bf16, host, rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from spark_engine_amd import ops
+    return ops
+
+
+def _stacked_mxfp4(ET, H, I, seed):
+    """expert tensors generated on the device (5 GB at 384 experts): uniform codes, scales 117..127"""
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    out = []
+    for rows, K in ((I, H), (I, H), (H, I)):
+        out.append(torch.randint(0, 256, (ET, rows, K // 2), dtype=torch.uint8, device=DEV, generator=g))
+        out.append(torch.randint(117, 128, (ET, rows, K // 32), dtype=torch.uint8, device=DEV, generator=g))
+    return out
+
+
+@pytest.mark.parametrize("R", [1, 2, 4])
+def test_c3_layer_full_shape_vs_oracle(ops, oracle, R):
+    # hidden 4096, intermediate 2048, top-6 + 1 shared, the full expert shape; 24 + 1 experts keep the host side small
+    H, I, E, topk, ns = 4096, 2048, 24, 6, 1
+    t = _stacked_mxfp4(E + ns, H, I, 31)
+    ex = ops.Mxfp4Experts(*t, n_shared=ns)
+    g = synth.rng(600 + R)
+    x = synth.randn_bf16(g, (R, H))
+    logits = g.standard_normal((R, E)).astype(np.float32)
+    idx, rw = oracle.ds41_route(logits, np.zeros(E, np.float32), topk, 1.5)
+    y = host(ops.mxfp4_moe_x(dev_bf16(x), dev(idx), dev(rw), ex))
+    ref = oracle.mxfp4_moe(x, idx, rw, *[host(a) for a in t], n_shared=ns)
+    assert rel_l2(y, ref) <= TOL, rel_l2(y, ref)
+
+
+@pytest.mark.parametrize("N,K", [(7168, 4096), (4096, 7168)])
+@pytest.mark.parametrize("R", [1, 4])
+def test_c4_projection_full_shape_vs_oracle(ops, oracle, N, K, R):
+    g = synth.rng(610 + R)
+    w8, s = synth.fp8_block_matrix(g, N, K)
+    x = synth.randn_bf16(g, (R, K))
+    y = host(ops.fp8_block128_gemv(dev_bf16(x), dev(w8), dev(s)))
+    ref = oracle.fp8_block_gemv(x, w8, s)
+    assert rel_l2(y, ref) <= 1e-5, rel_l2(y, ref)
+    # linear in the activations: a row scaled by a power of two scales its output exactly
+    x2 = synth.bf16_bits(synth.bf16_to_f32(x) * 4.0)
+    assert np.array_equal(host(ops.fp8_block128_gemv(dev_bf16(x2), dev(w8), dev(s))), y * 4.0)
+
+
+def test_c5_prefill_rows_equal_decode_rows(ops, oracle):
+    # 2048 tokens, 384 experts top-6, Zipf(1.1) routing, full shapes
+    H, I, E, topk, R = 4096, 2048, 384, 6, 2048
+    t = _stacked_mxfp4(E, H, I, 32)
+    ex = ops.Mxfp4Experts(*t)
+    g = synth.rng(620)
+    x = synth.randn_bf16(g, (R, H))
+    idx, rw = synth.zipf_routes(g, R, E, topk)
+    counts = np.bincount(idx.ravel(), minlength=E)
+    assert counts.max() > 512 and (counts > 0).sum() > 300              # heavy and light experts: several items per expert, ragged tails
+    xd, idxd, rwd = dev_bf16(x), dev(idx), dev(rw)
+    y = ops.mxfp4_moe(xd, idxd, rwd, ex)
+    torch.cuda.synchronize()
+    yh = host(y)
+    assert np.isfinite(yh).all()
+    hot = int(np.argmax(counts))
+    rows = [0, 777, R - 1, int(np.nonzero((idx == hot).any(1))[0][5]), int(np.nonzero((idx == int(np.argmin(np.where(counts > 0, counts, R))))
+                                                                                         .any(1))[0][0])]
+    for r in rows:                                                       # the same row alone, through the single-launch decode path
+        one = host(ops.mxfp4_moe_x(xd[r:r + 1], idxd[r:r + 1], rwd[r:r + 1], ex))
+        assert np.array_equal(one[0], yh[r]), r
+    for r in rows[:2]:                                                   # and against the oracle (only the row's experts go to the host)
+        used = sorted(set(idx[r].tolist()))
+        remap = {e: i for i, e in enumerate(used)}
+        sub = [host(a[used]) for a in t]
+        ref = oracle.mxfp4_moe(x[r:r + 1], np.array([[remap[e] for e in idx[r]]], np.int64), rw[r:r + 1], *sub)
+        assert rel_l2(yh[r:r + 1], ref) <= TOL
