@@ -105,6 +105,12 @@ SPARK_API int ds41_fp8_gemv_ex(const void* x, const void* w, const void* ws, flo
 SPARK_API int ds41_fp8_gemv(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, hipStream_t st);
 /* The same product for up to 16 rows.  Replaces engine-rs/shim/ds41_mx.cu:1385-1393 (ds41_fp8_gemv_bx). */
 SPARK_API int ds41_fp8_gemv_bx(const void* x, const void* w, const void* ws, float* y, int m, int n, int k, int xs, int rpg, hipStream_t st);
+/* FP8 weights times act-quantised activations, m <= 32: x bf16 [m, k] (quantised inside when aq is NULL) or aq E4M3 + as_ UE8M0
+ * per 32; y fp32, or bf16 when ob16.  Replace engine-rs/shim/ds41_mx.cu:1348-1382. */
+SPARK_API int ds41_fp8_gemv_mx_init(void);
+SPARK_API size_t ds41_fp8_gemv_mx_smem_max(void);
+SPARK_API int ds41_fp8_gemv_mx_q(const void* x, const void* aq, const void* as_, const void* w, const void* ws, void* y, int m, int n, int k,
+                                 int ob16, hipStream_t st);
 /* w [n, k] E4M3 with fp32 scales [ceil(n/128), ceil(k/128)]; the projection of reference/ds41/kernel.py:96-119 (fp8_gemm) with bf16
  * activations used as given. */
 SPARK_API int spark_fp8_block128_gemv(const void* x, const void* w, const float* scales, float* y, int m, int n, int k, hipStream_t st);

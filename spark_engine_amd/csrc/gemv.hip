@@ -134,6 +134,102 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void qgemv_kernel(const uint16_t* 
         }
 }
 
+// FP8 weights (E4M3 + E8M0 per 32 x 32) times act-quantised activations (E4M3 + UE8M0 per 32): the products are exact in
+// binary32, only the summation order is this kernel's.  The activations arrive quantised (aq, as) or as bf16 x, which the
+// workgroup quantises into LDS first with the rule of act_quant (the same bytes and scales as ds41_act_quant_fp8).
+// LDS: code values as bf16 [M][k] (exact) + scales as binary32 [M][k / 32].  reference ds41_mx.cu:953-1100 (fp8_gemv_mx).
+template <int M>
+__global__ __launch_bounds__(64 * GEMV_WAVES) void fp8q_gemv_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ aq, const uint8_t* __restrict__ as_,
+                                                                    const uint8_t* __restrict__ w, const uint8_t* __restrict__ ws, void* __restrict__ y, int ob16,
+                                                                    int m, int n, int k)
+{
+    extern __shared__ uint16_t xl[];                      // [M][k] bf16 code values, then [M][k / 32] binary32 scales
+    float* sx = (float*)(xl + (size_t)M * k);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nb32 = k >> 5;
+    for (int i = threadIdx.x; i < m * nb32 * 4; i += blockDim.x) {         // 4 threads per 32-block, 8 elements each
+        const int r = i / (nb32 * 4), q = i % (nb32 * 4), b = q >> 2, c = b * 32 + (q & 3) * 8;
+        uint32_t code[2], e;
+        if (aq) {
+            const uint2 v = *(const uint2*)(aq + (int64_t)r * k + c);
+            code[0] = v.x; code[1] = v.y;
+            e = as_[(int64_t)r * nb32 + b];
+        } else {
+            const uint4 raw = *(const uint4*)(x + (int64_t)r * k + c);
+            const uint32_t rw4[4] = {raw.x, raw.y, raw.z, raw.w};
+            float v[8], am = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[2 * j] = __uint_as_float(rw4[j] << 16); v[2 * j + 1] = __uint_as_float(rw4[j] & 0xffff0000u);
+                am = fmaxf(am, fmaxf(fabsf(v[2 * j]), fabsf(v[2 * j + 1])));
+            }
+            am = fmaxf(am, lane_xor<1>(am, lane));
+            am = fmaxf(am, lane_xor<2>(am, lane));
+            e = aq_scale(am);
+            code[0] = code[1] = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { code[0] |= aq_byte(v[j], e) << (8 * j); code[1] |= aq_byte(v[4 + j], e) << (8 * j); }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xl[(size_t)r * k + c + j] = f32_to_bf16(e4m3_to_f32((code[j >> 2] >> (8 * (j & 3))) & 0xffu));
+        if ((q & 3) == 0) sx[r * nb32 + b] = e8m0_to_f32(e);
+    }
+    __syncthreads();
+    const int row0 = blockIdx.x * (GEMV_WAVES * RPW) + wave * RPW;
+    if (row0 >= n) return;
+    float acc[RPW][M];
+#pragma unroll
+    for (int i = 0; i < RPW; ++i)
+#pragma unroll
+        for (int r = 0; r < M; ++r) acc[i][r] = 0.f;
+    for (int c = lane * 16; c < k; c += 64 * 16) {
+        uint4 p[RPW];
+        float s[RPW];
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const int row = row0 + i < n ? row0 + i : n - 1;
+            p[i] = ld_stream16(w + (int64_t)row * k + c);
+            s[i] = e8m0_to_f32(ws[(int64_t)(row >> 5) * nb32 + (c >> 5)]);
+        }
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const uint32_t pw[4] = {p[i].x, p[i].y, p[i].z, p[i].w};
+            bf2 wv[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                wv[2 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, false);
+                wv[2 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, true);
+            }
+#pragma unroll
+            for (int r = 0; r < M; ++r) {
+                if (r >= m) break;
+                const uint32_t* xp = (const uint32_t*)(xl + (size_t)r * k + c);
+                float t = 0.f;
+#pragma unroll
+                for (int j = 0; j < 8; j += 4) {
+                    const uint4 xv = *(const uint4*)(xp + j);
+                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 0], as_bf2(xv.x), t, false);
+                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 1], as_bf2(xv.y), t, false);
+                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 2], as_bf2(xv.z), t, false);
+                    t = __builtin_amdgcn_fdot2_f32_bf16(wv[j + 3], as_bf2(xv.w), t, false);
+                }
+                acc[i][r] = __builtin_fmaf(t, s[i] * sx[r * nb32 + (c >> 5)], acc[i][r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < RPW; ++i)
+#pragma unroll
+        for (int r = 0; r < M; ++r) {
+            if (r >= m) break;
+            const float v = wave_sum(acc[i][r]);
+            if (lane == 0 && row0 + i < n) {
+                if (ob16) ((uint16_t*)y)[(int64_t)r * n + row0 + i] = f32_to_bf16(v);
+                else ((float*)y)[(int64_t)r * n + row0 + i] = v;
+            }
+        }
+}
+
 template <int M>
 __global__ __launch_bounds__(64 * GEMV_WAVES) void bf16_gemv_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float* __restrict__ y,
                                                                     int m, int n, int k)
@@ -205,6 +301,35 @@ SPARK_API int ds41_fp8_gemv_ex(const void* x, const void* w, const void* ws, flo
 {
     if (m < 1 || m > 8 || n < 1 || k < 32 || k % 32 != 0 || (rpg && rpg % 32)) return 1;
     return launch_qgemv<1>(x, w, ws, y, m, n, k, xs, rpg, 0, st);
+}
+// x bf16 [m, k] (quantised inside when aq is null) or aq E4M3 [m, k] + as_ UE8M0 [m, k/32]; w E4M3 [n, k] + ws E8M0 per 32 x 32;
+// y [m, n] fp32, or bf16 when ob16; m <= 32 (rows beyond 8 take further passes of the same kernel: a row's value does not depend
+// on m).  reference ds41_mx.cu:1357-1380
+SPARK_API int ds41_fp8_gemv_mx_init() { return 0; }
+SPARK_API size_t ds41_fp8_gemv_mx_smem_max() { return 128 * 1024; }
+SPARK_API int ds41_fp8_gemv_mx_q(const void* x, const void* aq, const void* as_, const void* w, const void* ws, void* y, int m, int n, int k, int ob16,
+                                 hipStream_t st)
+{
+    if (m < 1 || m > 32 || k % 64 || n % 8 || (!x && !aq) || (aq && !as_)) return 1;
+    const dim3 g((n + GEMV_WAVES * RPW - 1) / (GEMV_WAVES * RPW)), b(64 * GEMV_WAVES);
+    for (int r0 = 0; r0 < m; r0 += 8) {
+        const int mm = m - r0 < 8 ? m - r0 : 8;
+        const uint16_t* xr = x && !aq ? (const uint16_t*)x + (int64_t)r0 * k : nullptr;
+        const uint8_t* qr = aq ? (const uint8_t*)aq + (int64_t)r0 * k : nullptr;
+        const uint8_t* sr = aq ? (const uint8_t*)as_ + (int64_t)r0 * (k / 32) : nullptr;
+        void* yr = ob16 ? (void*)((uint16_t*)y + (int64_t)r0 * n) : (void*)((float*)y + (int64_t)r0 * n);
+#define FQ(MM)                                                                                                                                          \
+    do {                                                                                                                                                \
+        const size_t sm = (size_t)MM * k * 2 + (size_t)MM * (k / 32) * 4;                                                                               \
+        if (sm > LDS_MAX) return 2;                                                                                                                     \
+        static bool attr = hipFuncSetAttribute((const void*)fp8q_gemv_kernel<MM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX) == hipSuccess; \
+        if (!attr) return 3;                                                                                                                            \
+        fp8q_gemv_kernel<MM><<<g, b, sm, st>>>(xr, qr, sr, (const uint8_t*)w, (const uint8_t*)ws, yr, ob16, mm, n, k);                                  \
+    } while (0)
+        switch (mm) { case 1: FQ(1); break; case 2: FQ(2); break; case 3: case 4: FQ(4); break; default: FQ(8); }
+#undef FQ
+    }
+    return launch_status();
 }
 // reference ds41_mx.cu:1385-1393: the same product for up to 16 rows (there a tensor-core kernel whose cost does not grow with m);
 // here rows beyond 8 take a second pass of the same kernel, so a row's value does not depend on m

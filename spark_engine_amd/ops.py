@@ -230,6 +230,16 @@ def fp8_gemv_bx(x, w, s, rpg=0):
     return y
 
 
+def fp8_gemv_mx(x, w, s, aq=None, as_=None, bf16_out=False):
+    """reference kern.rs fp8_gemv_mx / fp8_gemv_mx_bf16 (ds41_fp8_gemv_mx_q): FP8 weights x act-quantised activations, up to 32 rows;
+    x bf16 [m, k] is quantised inside unless the quantised pair (aq, as_) is given."""
+    m = (x if aq is None else aq).shape[0]
+    n, k = w.shape
+    y = torch.empty(m, n, dtype=torch.bfloat16 if bf16_out else torch.float32, device=w.device)
+    _ck(_lib().ds41_fp8_gemv_mx_q(_p(x), _p(aq), _p(as_), _p(_dev(w)), _p(_dev(s)), _p(y), m, n, k, int(bf16_out), _st()), "ds41_fp8_gemv_mx_q")
+    return y
+
+
 def fp8_block128_gemv(x, w, scales, y=None):
     m, k = x.shape
     n = w.shape[0]

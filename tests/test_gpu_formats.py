@@ -184,6 +184,28 @@ def test_fp8_gemv_bx_up_to_16_rows_and_groups(ops, oracle):
         assert rel_l2(yg[:, 64 * j:64 * j + 64], refj) < 1e-5
 
 
+def test_fp8_gemv_with_quantised_activations(ops, oracle):
+    # FP8 weights x act-quantised activations: every product is exact, the reference is the same sum in float64
+    g = synth.rng(151)
+    n, k, m = 256, 1024, 11
+    w8, _ = synth.fp8_block_matrix(g, n, k)
+    s8 = g.integers(110, 128, (n // 32, k // 32), dtype=np.uint8)
+    x = synth.randn_bf16(g, (m, k))
+    q, s = oracle.act_quant_fp8(x)
+    W = oracle.fp8_e8m0_dequant(w8, s8).astype(np.float64)
+    codes = torch.from_numpy(q.copy()).view(torch.float8_e4m3fn).to(torch.float64).numpy()          # library decode of E4M3
+    xq = codes * np.exp2(s.astype(np.float64) - 127.0).repeat(32, axis=1)
+    ref = xq @ W.T
+    y = host(ops.fp8_gemv_mx(dev_bf16(x), dev(w8), dev(s8)))
+    assert rel_l2(y, ref) <= 3e-5, rel_l2(y, ref)                        # the reference's probe threshold (fp8_probe.rs:43,51)
+    y2 = host(ops.fp8_gemv_mx(None, dev(w8), dev(s8), aq=dev(q), as_=dev(s)))
+    assert np.array_equal(y, y2)                                         # quantised inside = quantised by the caller
+    yb = host(ops.fp8_gemv_mx(dev_bf16(x), dev(w8), dev(s8), bf16_out=True))
+    assert np.array_equal(yb, synth.bf16_bits(y))
+    y1 = host(ops.fp8_gemv_mx(dev_bf16(x[3:4]), dev(w8), dev(s8)))
+    assert np.array_equal(y1[0], y[3])                                   # a row's value does not depend on the row count
+
+
 def test_gemv_rejects_bad_shapes(ops):
     x = torch.zeros(9, 64, dtype=torch.bfloat16, device=DEV)
     w = torch.zeros(8, 32, dtype=torch.uint8, device=DEV)
