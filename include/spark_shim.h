@@ -176,6 +176,8 @@ SPARK_API int ds41_moe(const void* xq, int R, const int64_t* idx, const float* r
  * 1 int64; act: 0 silu(g) * u, 1 the same after clamping g <= 10 and |u| <= 10; codebook 1 mcg, 2 mul1.  out fp32 [R, H].
  * flags bit 0: ws was prepared by spark_exl3_moe_ws_init and only ever used by this entry point (skips the clearing launch);
  * flags bit 1: force the several-kernel path.
+ * flags bit 2: tab has a tenth row, uint64 [E], with each expert's trellis width (3..6 bits, engine-rs/shim/moe_exl3.cuh:239-252); all
+ * three matrices of an expert share it.  Runs on the several-kernel path.
  * Replaces engine-rs/shim/moe_exl3.cuh:1512-1691 (moex::experts). */
 SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk);
 SPARK_API int spark_exl3_moe_ws_init(void* ws, size_t bytes, hipStream_t st);
@@ -186,7 +188,8 @@ SPARK_API int spark_exl3_moe(const void* x, int xtype, int64_t ldx, int R, const
 SPARK_API size_t qwen_moe_ws_bytes(int R, int S);
 SPARK_API int qwen_moe_experts(const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out,
                                void* ws, int S, hipStream_t st);
-/* GLM: E 288, top-8, H 4096, I 1024, x / w fp16, idx int64, mcg, clamped activation; kmask must be 1 << 4 (4-bit experts only).
+/* GLM: E 288, top-8, H 4096, I 1024, x / w fp16, idx int64, mcg, clamped activation.  kmask = set of trellis widths present (bit b = some
+ * expert has b bits, 3..6): 1 << 4 reads a nine-row table of 4-bit experts, anything else a ten-row table (see spark_exl3_moe flags bit 2).
  * Replaces engine-rs/shim/glm_moe.cu:8-16. */
 SPARK_API size_t glm_moe_ws_bytes(int R, int S);
 SPARK_API int glm_moe_experts(const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out,

@@ -147,6 +147,67 @@ __global__ __launch_bounds__(64 * GV_WAVES) void gemv_kernel(const uint16_t* __r
     }
 }
 
+// Grouped GEMV for tables with mixed trellis widths (row 9 of the table = the expert's bits, 3..6; reference moe_exl3.cuh:239-252):
+// the same grid and outputs as gemv_kernel.  A k-tile's 16 x 128 strip is decoded into LDS with the generic state extraction
+// (the code of the dequantisation surface) and multiplied in binary32; thread = output column for the even or the odd item rows.
+template <int CBK>
+__global__ __launch_bounds__(256) void gemv_anybits_kernel(const uint16_t* __restrict__ xh, const uint64_t* __restrict__ tab, int E, int tr_slot0,
+                                                          const int* __restrict__ G, const int* __restrict__ gexp, const int* __restrict__ goff,
+                                                          const int* __restrict__ gcnt, int Gmax, int T, int P, int K, int N, int kts,
+                                                          float* __restrict__ part)
+{
+    __shared__ uint16_t wl[16 * 128];
+    __shared__ uint32_t tw[8 * 48];
+    const int tg = blockIdx.z, t = tg / Gmax, g = tg % Gmax;
+    if (g >= *G) return;
+    const int rows = gcnt[g], e = gexp[g];
+    const int bits = (int)tab[(int64_t)9 * E + e], nw = 8 * bits;
+    const int tid = threadIdx.x, col = tid & 127, half = tid >> 7;
+    const int Nt = N / 16, nb = blockIdx.x, s = blockIdx.y;
+    const uint32_t* tr = (const uint32_t*)tab[(int64_t)(tr_slot0 + t) * E + e];
+    const int64_t r0 = (int64_t)t * P + goff[g];
+    const uint16_t* xbase = xh + r0 * K;
+    const int kt0 = s * kts, kt1 = min(K / 16, kt0 + kts);
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+    if (bits >= 3 && bits <= 6)
+        for (int kt = kt0; kt < kt1; ++kt) {
+            __syncthreads();
+            for (int i = tid; i < 8 * nw; i += 256) tw[(i / nw) * 48 + i % nw] = tr[((int64_t)kt * Nt + nb * 8 + i / nw) * nw + i % nw];
+            __syncthreads();
+            for (int i = tid; i < 8 * 256; i += 256) {
+                const int tl = i >> 8, p = i & 255;
+                int row, c;
+                tile_pos(p, row, c);
+                const _Float16 v = cb_decode<CBK>(tile_state(tw + tl * 48, bits, p));
+                uint16_t hb; __builtin_memcpy(&hb, &v, 2);
+                wl[row * 128 + tl * 16 + c] = hb;
+            }
+            __syncthreads();
+            float wv[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) wv[r] = f16_bits_to_f32(wl[r * 128 + col]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int m = 2 * i + half;
+                if (m < rows) {
+                    const uint16_t* xr = xbase + (int64_t)m * K + kt * 16;
+                    float a = acc[i];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) a = __builtin_fmaf(f16_bits_to_f32(xr[r]), wv[r], a);
+                    acc[i] = a;
+                }
+            }
+        }
+    float* out = part + (((int64_t)s * T * P) + r0) * N + nb * 128;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int m = 2 * i + half;
+        if (m < rows) out[(int64_t)m * N + col] = acc[i];
+    }
+}
+
 // ---------------------------------------------------------------- mid: finish gate and up, act, down input transform
 // wave per (compact row, 128-block of I); reference moe_exl3.cuh:1019-1064
 __global__ __launch_bounds__(256) void mid_kernel(const float* __restrict__ part, int S, const uint64_t* __restrict__ tab, int E, int P, int I, int act,
@@ -238,10 +299,14 @@ inline bool cfg_ok(const Cfg& c, int R)
 
 template <int CBK>
 void launch_gemv(const uint16_t* xh, const uint64_t* tab, int E, int slot0, const int* G, const int* gexp, const int* goff, const int* gcnt, int Gmax, int T,
-                 int P, int K, int N, int S, int maxrows, float* part, hipStream_t st)
+                 int P, int K, int N, int S, int maxrows, float* part, hipStream_t st, bool mixed = false)
 {
     const dim3 grid(N / 128, S, T * Gmax), blk(64 * GV_WAVES);
     const int kts = (K / 16 + S - 1) / S;
+    if (mixed) {                                     // per-expert trellis widths from row 9 of the table
+        gemv_anybits_kernel<CBK><<<grid, 256, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
+        return;
+    }
     // one instantiation per row-count class of the call (items never hold more rows than the call has)
     if (maxrows <= 1) gemv_kernel<CBK, 1><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
     else if (maxrows <= 2) gemv_kernel<CBK, 2><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
@@ -250,13 +315,14 @@ void launch_gemv(const uint16_t* xh, const uint64_t* tab, int E, int slot0, cons
     else gemv_kernel<CBK, 16><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
 }
 
-// flags: bit 0 = the workspace counters are known to be zero (zeroed once, then only used by these calls);
-//        bit 1 = force the multi-kernel path
+// flags: bit 0 = the workspace is prepared (once, then only used by these calls);
+//        bit 1 = force the multi-kernel path; bit 2 = mixed trellis widths (table row 9 = bits per expert; multi-kernel path)
 int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
             int flags, hipStream_t st)
 {
     if (!cfg_ok(c, R)) return -1;
-    if (!(flags & 2) && exl3_fused_ok(c, R)) return exl3_fused_launch(c, x, ldx, R, idx, w, tab, add, out, ws, flags & 1, st);
+    const bool mixed = (flags & 4) != 0;             // the table has a row 9 with every expert's trellis width (3..6 bits)
+    if (!(flags & 2) && !mixed && exl3_fused_ok(c, R)) return exl3_fused_launch(c, x, ldx, R, idx, w, tab, add, out, ws, flags & 1, st);
     const Plan p = plan(c, R);
     char* b = (char*)ws + (exl3_fused_ok(c, R) ? exl3_fused_ws_bytes(c, R) : 0);       // the two paths never share workspace bytes
     int* G = (int*)(b + p.G);
@@ -270,12 +336,12 @@ int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, co
     prep_kernel<<<1, EMAX, 0, st>>>(idx, c.itype, R, c.topk, c.E, GR, G, gexp, goff, gcnt, pairmap, prow, pexp);
     int waves = 2 * p.P * (c.H / 128);
     had_kernel<<<(waves + 3) / 4, 256, 0, st>>>(x, c.xtype, ldx, tb, c.E, 3, 2, p.P, prow, pexp, c.H, xh1);
-    if (c.cbk == CB_MCG) launch_gemv<CB_MCG>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, p.S1, maxrows, part, st);
-    else launch_gemv<CB_MUL1>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, p.S1, maxrows, part, st);
+    if (c.cbk == CB_MCG) launch_gemv<CB_MCG>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, p.S1, maxrows, part, st, mixed);
+    else launch_gemv<CB_MUL1>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, p.S1, maxrows, part, st, mixed);
     waves = p.P * (c.I / 128);
     mid_kernel<<<(waves + 3) / 4, 256, 0, st>>>(part, p.S1, tb, c.E, p.P, c.I, c.act, pexp, xh2);
-    if (c.cbk == CB_MCG) launch_gemv<CB_MCG>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, p.S2, maxrows, part, st);
-    else launch_gemv<CB_MUL1>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, p.S2, maxrows, part, st);
+    if (c.cbk == CB_MCG) launch_gemv<CB_MCG>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, p.S2, maxrows, part, st, mixed);
+    else launch_gemv<CB_MUL1>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, p.S2, maxrows, part, st, mixed);
     waves = R * (c.H / 128);
     finish_combine_kernel<<<(waves + 3) / 4, 256, 0, st>>>(part, p.S2, tb, c.E, p.P, c.H, c.topk, pairmap, pexp, w, c.wtype, (const float*)add, (float*)out, R);
     return launch_status();
@@ -322,12 +388,13 @@ SPARK_API int qwen_moe_experts(const void* x, int64_t ldx, int R, const void* id
     return experts(QWEN, x, ldx, R, idx, w, tab, add, out, ws, 0, st);
 }
 // reference glm_moe.cu:6-24: x f16 [R, 4096], idx i64 / w f16 [R, 8], tab u64 [10|11][288] (rows 0-8 as above), mcg codebook,
-// clamped SwiGLU.  suh0 (shared gate/up input scales) is a prefill shortcut and is not needed; kmask must be 1 << 4.
+// clamped SwiGLU.  suh0 (shared gate/up input scales) is a prefill shortcut and is not needed.  kmask = bit K set for every
+// trellis width K present: 1 << 4 runs the 4-bit kernels, anything else reads every expert's width from row 9 of the table.
 SPARK_API size_t glm_moe_ws_bytes(int R, int S) { (void)S; return spark_exl3_moe_ws_bytes(R, GLM.H, GLM.I, GLM.E, GLM.topk); }
 SPARK_API int glm_moe_experts(const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws, int S,
                               const void* suh0, int kmask, hipStream_t st)
 {
     (void)S; (void)suh0;
-    if (kmask != (1 << 4)) return -4;                          // mixed trellis widths: not built
-    return experts(GLM, x, ldx, R, idx, w, tab, add, out, ws, 0, st);
+    if (kmask <= 0 || (kmask & ~0x78)) return -4;              // widths 3..6 only
+    return experts(GLM, x, ldx, R, idx, w, tab, add, out, ws, kmask == (1 << 4) ? 0 : 4, st);
 }

@@ -116,6 +116,60 @@ def test_single_launch_and_multi_kernel_paths_agree(ops, oracle, R):
         assert rel_l2(a, b) <= 3e-4                                      # fp16 roundings of the transformed activations can flip with the summation order
 
 
+@pytest.mark.parametrize("R", [1, 5])
+def test_mixed_trellis_widths(ops, oracle, R):
+    # every expert with its own trellis width, 3..6 bits, in row 9 of the table (reference moe_exl3.cuh:239-252)
+    g = synth.rng(460 + R)
+    H, I, E, topk = 512, 256, 8, 3
+    bits = {e: 3 + e % 4 for e in range(E)}
+    experts = {e: synth.exl3_expert(g, H, I, bits[e]) for e in range(E)}
+    table = ops.ExpertTable(_to_dev(experts), E, bits=bits)
+    assert table.kmask == 0x78
+    idx = np.stack([g.permutation(E)[:topk] for _ in range(R)]).astype(np.int32)
+    w = g.uniform(0.1, 1.0, (R, topk)).astype(np.float32)
+    xb = synth.randn_bf16(g, (R, H))
+    out = host(ops.exl3_moe(dev_bf16(xb), dev(idx), dev(w), table, H, I))
+    # the oracle takes one width per call: one pass per width with the other experts' pairs weighted 0 (their tables replaced by
+    # zero codes of that width), summed
+    ref = np.zeros((R, H), np.float32)
+    for b in (3, 4, 5, 6):
+        ex_b = {e: (experts[e] if bits[e] == b else tuple(np.zeros_like(synth.exl3_expert(synth.rng(1), H, I, b)[s]) if s < 3 else experts[e][s] for s in range(9)))
+                for e in range(E)}
+        w_b = np.where(np.vectorize(bits.get)(idx) == b, w, 0.0).astype(np.float32)
+        ref += oracle.exl3_moe(synth.bf16_to_f32(xb), idx, w_b, ex_b, E, H, I, b, 2, 0)
+    assert rel_l2(out, ref) <= TOL, rel_l2(out, ref)
+    # all-4-bit experts through the same kernel agree with the 4-bit kernels
+    ex4 = {e: synth.exl3_expert(g, H, I, 4) for e in range(E)}
+    t4m = ops.ExpertTable(_to_dev(ex4), E, bits={e: 4 for e in range(E)})
+    t4 = ops.ExpertTable(_to_dev(ex4), E)
+    a = host(ops.exl3_moe(dev_bf16(xb), dev(idx), dev(w), t4m, H, I))
+    b4 = host(ops.exl3_moe(dev_bf16(xb), dev(idx), dev(w), t4, H, I))
+    assert rel_l2(a, b4) <= 3e-4
+
+
+def test_glm_mixed_widths_through_kmask(ops, oracle):
+    # GLM's entry point with kmask naming 3- and 4-bit experts (the reference's mixed checkpoint tables)
+    g = synth.rng(470)
+    R, E, H, I = 1, 288, 4096, 1024
+    idx8 = g.permutation(E)[:8].astype(np.int64)[None]
+    bits = {int(e): 3 + (k & 1) for k, e in enumerate(idx8[0])}
+    experts = {e: synth.exl3_expert(g, H, I, b) for e, b in bits.items()}
+    w8 = (g.uniform(0, 1, (R, 8)) + 0.1).astype(np.float16)
+    x16 = g.standard_normal((R, H)).astype(np.float16)
+    t = ops.ExpertTable(_to_dev(experts), E, bits=bits)
+    assert t.kmask == (1 << 3 | 1 << 4)
+    out = host(ops.glm_moe_experts(dev_f16(x16.view(np.uint16)), dev(idx8), dev_f16(w8.view(np.uint16)), t, kmask=t.kmask))
+    ref = np.zeros((R, H), np.float32)
+    for b in (3, 4):
+        sel = {e: experts[e] for e in experts if bits[e] == b}
+        w_b = np.where(np.vectorize(bits.get)(idx8) == b, w8.astype(np.float32), 0.0).astype(np.float32)
+        idx_b = np.where(np.vectorize(bits.get)(idx8) == b, idx8, next(iter(sel))).astype(np.int32)
+        ref += oracle.exl3_moe(x16.astype(np.float32), idx_b, w_b, sel, E, H, I, b, 1, 1)
+    assert rel_l2(out, ref) <= TOL
+    with pytest.raises(RuntimeError):
+        ops.glm_moe_experts(dev_f16(x16.view(np.uint16)), dev(idx8), dev_f16(w8.view(np.uint16)), t, kmask=1 << 7)
+
+
 def test_exl3_moe_rejects_bad_shapes(ops):
     x = torch.zeros(1, 200, device=DEV)
     with pytest.raises(ops.KernelError):
