@@ -197,8 +197,10 @@ SPARK_API int glm_moe_experts(const void* x, int64_t ldx, int R, const void* idx
 
 /* ---------------------------------------------------------------- diagnostics (not part of the reference ABI) ---------------- */
 
-/* buf = device memory of 8 * gridDim int64 the single-launch EXL3 kernel fills with per-block wall-clock stamps (NULL = off) */
+/* buf = device memory of 16 * gridDim int64 the single-launch kernels fill with per-block wall-clock stamps (NULL = off).  Only
+ * libraries built with -DSPK_EXL3_TRACE / -DSPK_MX_TRACE record stamps; the release build ignores the buffer. */
 SPARK_API void spark_debug_exl3_trace(long long* buf);
+SPARK_API void spark_debug_mx_trace(long long* buf);
 /* exchange mode of the single-launch EXL3 kernel: 1 = same-XCD through L2, 0 = device-coherent, -1 = measure placement again */
 SPARK_API void spark_debug_exl3_local(int v);
 

@@ -14,6 +14,11 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
 
+# extra compiler flags for diagnostic builds, e.g. SPARK_HIPCC_EXTRA="-DSPK_EXL3_TRACE -DSPK_MX_TRACE" (per-block time stamps
+# of the single-launch kernels, read through spark_debug_exl3_trace / spark_debug_mx_trace)
+EXTRA = os.environ.get("SPARK_HIPCC_EXTRA", "").split()
+
+
 def sources():
     return sorted(CSRC.glob("*.hip")) + sorted(CSRC.glob("*.cpp"))
 
@@ -25,7 +30,7 @@ def build(verbose=False):
 
     def cc(src):
         obj = objdir / (src.stem + ".o")
-        cmd = [HIPCC, *FLAGS, "-c", str(src), "-o", str(obj)]
+        cmd = [HIPCC, *FLAGS, *EXTRA, "-c", str(src), "-o", str(obj)]
         if src.suffix == ".cpp":
             cmd = [HIPCC, "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-x", "c++", "-c", str(src), "-o", str(obj)]
         r = subprocess.run(cmd, capture_output=True, text=True)

@@ -38,10 +38,14 @@ namespace spk {
 namespace {
 
 long long* g_trace = nullptr;
-#define TRACE(i) do { if (a.trace && tid == 0) a.trace[(int64_t)bid * 8 + (i)] = wall_clock64(); } while (0)
+#ifdef SPK_EXL3_TRACE
+#define TRACE(i) do { if (a.trace && tid == 0) a.trace[(int64_t)bid * 16 + (i)] = wall_clock64(); } while (0)
+#else
+#define TRACE(i) do { } while (0)
+#endif
 
 constexpr int FW = 4;                 // waves per block
-constexpr int TWB = 8;                // k-tiles per wave of a stage-2 block (all loaded up front): K slice of 512
+constexpr int TWB = 4;                // k-tiles per wave of a stage-2 block (all loaded up front): K slice of 512
 constexpr int TWMAX = 8;              // most k-tiles per wave of a stage-1 block (4 or 8, chosen per shape)
 constexpr int PF_MAX = 256, RF_MAX = 16;
 constexpr int SPIN_MAX = 200000;
@@ -166,7 +170,7 @@ __device__ __forceinline__ Group find_item(const FArgs& a, int g, int* sidx, uns
 }
 
 template <int CBK, int MR, int TWA, bool LOCAL>
-__global__ __launch_bounds__(64 * FW) void fused_kernel(const FArgs a)
+__global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
 {
     __shared__ __align__(16) uint16_t xs[MR][FW * TWMAX * 16];   // this block's K slice of the transformed activations (fp16)
     __shared__ float red[FW][MR][128];

@@ -28,6 +28,13 @@ namespace {
 
 struct Item { int e, off, n, pad; };
 
+#ifdef SPK_MX_TRACE
+__device__ long long* g_gtrace = nullptr;     // 16 stamps per block of up_res_kernel
+#define GTRACE(i) do { if (g_gtrace && threadIdx.x == 0) { const int64_t bb = (int64_t)blockIdx.y * gridDim.x + blockIdx.x; if (bb < 32768) g_gtrace[bb * 16 + (i)] = wall_clock64(); } } while (0)
+#else
+#define GTRACE(i) do { } while (0)
+#endif
+
 constexpr int EMAXG = 2048;            // experts the grouping kernel can hold
 constexpr int UP_WAVES = 8, DN_WAVES = 4;
 
@@ -232,6 +239,381 @@ __global__ __launch_bounds__(64 * DN_WAVES) void down_kernel(const uint8_t* __re
     }
 }
 
+// ---------------------------------------------------------------- the same two products for shapes whose K groups all fit the
+// block's waves (one K group per wave): the weight rows stay in registers for every group of 16 item rows, and the loop is
+// software-pipelined - the next row group's activations (and the row bookkeeping of the one after) are requested right after
+// this group's MFMAs have consumed their operands, so their latency hides behind the reduction and the epilogue.  Same MFMA
+// and summation order as up_kernel / down_kernel: the same bits.
+template <int LAYOUT>
+__global__ __launch_bounds__(64 * UP_WAVES, 4) void up_res_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, WMat w1, WMat w3, int H, int I,
+                                                                  int TT, const int* __restrict__ G, const Item* __restrict__ items,
+                                                                  const int* __restrict__ prow, const float* __restrict__ pw, uint8_t* __restrict__ hq,
+                                                                  uint8_t* __restrict__ hs)
+{
+    __shared__ float red[UP_WAVES][4][4][64];      // [wave][tile: g0 g1 u0 u1][v][lane]
+    __shared__ float amx[UP_WAVES][16];
+    if ((int)blockIdx.y >= *G) return;
+    GTRACE(0);
+    const Item it = items[blockIdx.y];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, rg = lane >> 4;
+    const int j0 = blockIdx.x * 32;
+    const int steps = H >> 7, nkg = (steps + 3) >> 2;
+    const bool active = wave < nkg;
+    const int kg = active ? wave : 0;
+    // rows past the item's end repeat its last row (no branch around a load); their results are not stored
+    int pos = it.off + min(c, it.n - 1);
+    int tok = prow[pos] / TT;
+    float wgt = pw[pos];
+    int posn = it.off + min(16 + c, it.n - 1);
+    int tokn = prow[posn] / TT;
+    float wgtn = pw[posn];
+    v4i a[4][4];
+    uint32_t sa[4];
+    load_group<LAYOUT>(w1, it.e, j0, kg, lane, a[0], sa[0]);
+    load_group<LAYOUT>(w1, it.e, j0 + 16, kg, lane, a[1], sa[1]);
+    load_group<LAYOUT>(w3, it.e, j0, kg, lane, a[2], sa[2]);
+    load_group<LAYOUT>(w3, it.e, j0 + 16, kg, lane, a[3], sa[3]);
+    GTRACE(1);
+    const int ncg = (it.n + 15) >> 4;
+    for (int cg = 0; cg < ncg; ++cg) {
+        v4f acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) { acc[t] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(acc[t])); }
+        if (active) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                if (kg * 4 + s >= steps) break;
+                v8i b; uint32_t sb;
+#ifndef SPK_EXP_NOX
+                load_b(xq + (int64_t)tok * H, xs + (int64_t)tok * (H >> 5), kg * 4 + s, lane, b, sb);
+#else
+                b = v8i{tok, s, lane, cg, 1, 2, 3, 4}; sb = 127;
+#endif
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[t] = mfma_group_step(s, a[t][s], b, acc[t], sa[t], sb);
+            }
+        }
+        if (cg < 3) GTRACE(2 + cg * 4);
+        // the next row group's operands, and the rows of the one after
+        const int pos2 = it.off + min((cg + 2) * 16 + c, it.n - 1);
+        const int tok2 = prow[pos2] / TT;
+        const float wgt2 = pw[pos2];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][t][v][lane] = acc[t][v];
+        if (cg < 3) GTRACE(3 + cg * 4);
+        __syncthreads();
+        if (cg < 3) GTRACE(4 + cg * 4);
+        // epilogue: thread (wave = (tp, v), lane = (c, rg)) owns feature j0 + 16 tp + 4 rg + v of column c
+        const bool valid = cg * 16 + c < it.n;
+        const int tp = wave >> 2, v = wave & 3;
+        float gsum = 0.f, usum = 0.f;
+#pragma unroll
+        for (int w = 0; w < UP_WAVES; ++w) { gsum += red[w][tp][v][lane]; usum += red[w][2 + tp][v][lane]; }
+        const float gt = fminf(bf16_round(gsum), 10.f);
+        const float up = fminf(fmaxf(bf16_round(usum), -10.f), 10.f);
+        const float yv = bf16_round(silu(gt) * up * (valid ? wgt : 0.f));
+        float am = fabsf(yv);
+        am = fmaxf(am, __shfl_xor(am, 16, 64));
+        am = fmaxf(am, __shfl_xor(am, 32, 64));
+        if (rg == 0) amx[wave][c] = am;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < UP_WAVES; ++w) am = fmaxf(am, amx[w][c]);
+        const uint32_t e = aq_scale(am);
+#ifndef SPK_EXP_NOST
+        if (valid) {
+            hq[(int64_t)pos * I + j0 + 16 * tp + 4 * rg + v] = (uint8_t)aq_byte(yv, e);
+            if (wave == 0 && rg == 0) hs[(int64_t)pos * (I >> 5) + (j0 >> 5)] = (uint8_t)e;
+        }
+#else
+        if (valid && e == 0x12345u) hq[0] = (uint8_t)aq_byte(yv, e);
+#endif
+        __syncthreads();
+        pos = posn; tok = tokn; wgt = wgtn; posn = pos2; tokn = tok2; wgtn = wgt2;
+    }
+}
+
+template <int LAYOUT>
+__global__ __launch_bounds__(64 * DN_WAVES) void down_res_kernel(const uint8_t* __restrict__ hq, const uint8_t* __restrict__ hs, WMat w2, int H, int I,
+                                                                 const int* __restrict__ G, const Item* __restrict__ items, float* __restrict__ out)
+{
+    __shared__ float red[DN_WAVES][2][4][64];
+    if ((int)blockIdx.y >= *G) return;
+    const Item it = items[blockIdx.y];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15;
+    const int n0 = blockIdx.x * 32;
+    const int steps = I >> 7, nkg = (steps + 3) >> 2;
+    const bool active = wave < nkg;
+    const int kg = active ? wave : 0;
+    v4i a[2][4];
+    uint32_t sa[2];
+    load_group<LAYOUT>(w2, it.e, n0, kg, lane, a[0], sa[0]);
+    load_group<LAYOUT>(w2, it.e, n0 + 16, kg, lane, a[1], sa[1]);
+    v8i b[4];
+    uint32_t sb[4];
+    {
+        const int pos = it.off + min(c, it.n - 1);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) load_b(hq + (int64_t)pos * I, hs + (int64_t)pos * (I >> 5), min(kg * 4 + s, steps - 1), lane, b[s], sb[s]);
+    }
+    const int ncg = (it.n + 15) >> 4;
+    for (int cg = 0; cg < ncg; ++cg) {
+        const int rr = cg * 16 + c;
+        const int pos = it.off + min(rr, it.n - 1);
+        v4f acc[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) { acc[t] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(acc[t])); }
+        if (active) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                if (kg * 4 + s >= steps) break;
+#pragma unroll
+                for (int t = 0; t < 2; ++t) acc[t] = mfma_group_step(s, a[t][s], b[s], acc[t], sa[t], sb[s]);
+            }
+        }
+        {
+            const int posn = it.off + min(rr + 16, it.n - 1);      // the next row group's operands
+#pragma unroll
+            for (int s = 0; s < 4; ++s) load_b(hq + (int64_t)posn * I, hs + (int64_t)posn * (I >> 5), min(kg * 4 + s, steps - 1), lane, b[s], sb[s]);
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][t][v][lane] = acc[t][v];
+        __syncthreads();
+        // thread (wave = v, lane) sums both tiles' element v
+        const int v = wave, rg = lane >> 4;
+        if (rr < it.n) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                float sm = 0.f;
+#pragma unroll
+                for (int w = 0; w < DN_WAVES; ++w) sm += red[w][t][v][lane];
+                out[(int64_t)pos * H + n0 + 16 * t + 4 * rg + v] = sm;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------- prefill: grouped GEMM over 32-row items (T16 records)
+// Many rows per expert make the products above re-read every item's activation rows once per 32 output features and write the
+// intermediate in single bytes; both cost more than the weight stream.  Here a block owns 32 item rows x 128 output features
+// for the whole K range: the item's activation rows go through LDS one K group (512) at a time, double-buffered and shared by
+// the 8 waves (wave = 16 features, both matrices, two 16-row tiles), the weight records stream straight from memory into the
+// MFMA A operand through a four-step register ring that is refilled as soon as a step's MFMAs are issued, and results leave in
+// whole 128-byte lines.  Each K group accumulates from zero and the groups are added in order: the values are the same bits as
+// up_kernel / down_kernel and the single-launch kernel produce (reference engine-rs/shim/ds41_mx.cu:694-932 keeps the same
+// property between its grouped GEMM and its decode kernels).
+constexpr int GT_ROWS = 32;            // rows of a GEMM item
+constexpr int GT_XS = 528;             // LDS stride of a staged row: one K group (512 bytes) + 16: conflict-free 16-byte reads down a column
+constexpr int GT_FEAT = 128;           // output features / columns of a block
+
+__device__ __forceinline__ v4i ld_a_step(const uint8_t* rec, int s, int lane)
+{
+    const uint4 v = ld_stream16(rec + s * 1024 + lane * 16);
+    return v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+}
+__device__ __forceinline__ uint32_t ld_a_scales(const uint8_t* rec, int lane) { return __builtin_nontemporal_load((const uint32_t*)(rec + 4096 + lane * 4)); }
+
+__global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, WMat w1, WMat w3, int H, int I, int TT,
+                                                         const int* __restrict__ G, const Item* __restrict__ items, const int* __restrict__ prow,
+                                                         const float* __restrict__ pw, uint8_t* __restrict__ hq, uint8_t* __restrict__ hs)
+{
+    __shared__ __align__(16) unsigned char xl[2][GT_ROWS * GT_XS];
+    __shared__ __align__(16) unsigned char xsl[2][GT_ROWS * 16];
+    __shared__ int toks[GT_ROWS];
+    __shared__ float wgts[GT_ROWS];
+    __shared__ float amx[8][2][16];
+    __shared__ __align__(16) unsigned char hbuf[GT_ROWS][GT_FEAT + 16];
+    __shared__ __align__(4) unsigned char hes[GT_ROWS][4];
+    if ((int)blockIdx.y >= *G) return;
+    const Item it = items[blockIdx.y];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, rg = lane >> 4;
+    const int f0 = blockIdx.x * GT_FEAT;
+    const int nkg = H >> 9;
+    const int nrt = (it.n + 15) >> 4;
+    if (tid < GT_ROWS) {
+        const int pos = it.off + min(tid, it.n - 1);
+        toks[tid] = prow[pos] / TT;
+        wgts[tid] = tid < it.n ? pw[pos] : 0.f;
+    }
+    // the wave's weight records: 16 gate and 16 up rows, K group 0 first
+    const int64_t tile = ((int64_t)it.e * I + f0 + 16 * wave) >> 4;
+    const uint8_t* r1 = w1.w + tile * nkg * REC;
+    const uint8_t* r3 = w3.w + tile * nkg * REC;
+    v4i a[2][4];
+    uint32_t sa[2];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) { a[0][s] = ld_a_step(r1, s, lane); a[1][s] = ld_a_step(r3, s, lane); }
+    sa[0] = ld_a_scales(r1, lane); sa[1] = ld_a_scales(r3, lane);
+    __syncthreads();
+    // staging: thread = (row, 32-byte chunk) of a K group; threads 0..31 also carry the row's 16 scale bytes
+    const int srow = tid >> 4, sch = tid & 15;
+    const uint8_t* xrow = xq + (int64_t)toks[srow] * H + sch * 32;
+    const uint8_t* xsrow = xs + (int64_t)toks[tid & (GT_ROWS - 1)] * (H >> 5);
+    unsigned char* const xdst = &xl[0][srow * GT_XS + sch * 32];
+    uint4 x0 = *(const uint4*)xrow, x1 = *(const uint4*)(xrow + 16), xsc = *(const uint4*)xsrow;
+    *(uint4*)xdst = x0; *(uint4*)(xdst + 16) = x1;
+    if (tid < GT_ROWS) *(uint4*)&xsl[0][tid * 16] = xsc;
+    {
+        const int k1 = min(1, nkg - 1);
+        x0 = *(const uint4*)(xrow + k1 * 512); x1 = *(const uint4*)(xrow + k1 * 512 + 16); xsc = *(const uint4*)(xsrow + k1 * 16);
+    }
+    __syncthreads();
+    v4f tot[2][2];
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) tot[m][rt] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int kg = 0; kg < nkg; ++kg) {
+        const int buf = kg & 1, kn = min(kg + 1, nkg - 1);
+        const uint8_t* n1 = r1 + (int64_t)kn * REC;
+        const uint8_t* n3 = r3 + (int64_t)kn * REC;
+        const uint32_t san0 = ld_a_scales(n1, lane), san1 = ld_a_scales(n3, lane);
+        v4f cur[2][2];
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) { cur[m][rt] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(cur[m][rt])); }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                if (rt < nrt) {
+                    const unsigned char* bp = &xl[buf][(rt * 16 + c) * GT_XS + s * 128 + 16 * rg];
+                    const uint4 lo = *(const uint4*)bp, hi = *(const uint4*)(bp + 64);
+                    const v8i b = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+                    const uint32_t sb = *(const uint32_t*)&xsl[buf][(rt * 16 + c) * 16 + s * 4] >> (8 * rg);
+                    cur[0][rt] = mfma_group_step(s, a[0][s], b, cur[0][rt], sa[0], sb);
+                    cur[1][rt] = mfma_group_step(s, a[1][s], b, cur[1][rt], sa[1], sb);
+                }
+            }
+            a[0][s] = ld_a_step(n1, s, lane);          // the ring slot is free again: the same step of the next K group
+            a[1][s] = ld_a_step(n3, s, lane);
+        }
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) tot[m][rt] += cur[m][rt];
+        sa[0] = san0; sa[1] = san1;
+        // the next K group of the rows into the other buffer (nobody reads it before the barrier), the one after into registers
+        unsigned char* d = xdst + (buf ^ 1) * (GT_ROWS * GT_XS);
+        *(uint4*)d = x0; *(uint4*)(d + 16) = x1;
+        if (tid < GT_ROWS) *(uint4*)&xsl[buf ^ 1][tid * 16] = xsc;
+        const int k2 = min(kg + 2, nkg - 1);
+        x0 = *(const uint4*)(xrow + k2 * 512); x1 = *(const uint4*)(xrow + k2 * 512 + 16); xsc = *(const uint4*)(xsrow + k2 * 16);
+        __syncthreads();
+    }
+    // ---- SwiGLU * route weight, act_quant per 32 features (this wave's 16 and its neighbour's), 128 code bytes + 4 scales per row
+    float yv[2][4];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        const float wgt = wgts[rt * 16 + c];
+        float am = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float gt = fminf(bf16_round(tot[0][rt][i]), 10.f);
+            const float up = fminf(fmaxf(bf16_round(tot[1][rt][i]), -10.f), 10.f);
+            yv[rt][i] = bf16_round(silu(gt) * up * wgt);
+            am = fmaxf(am, fabsf(yv[rt][i]));
+        }
+        am = fmaxf(am, __shfl_xor(am, 16, 64));
+        am = fmaxf(am, __shfl_xor(am, 32, 64));
+        if (rg == 0) amx[wave][rt][c] = am;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        const uint32_t e = aq_scale(fmaxf(amx[wave][rt][c], amx[wave ^ 1][rt][c]));
+        uint32_t word = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) word |= aq_byte(yv[rt][i], e) << (8 * i);
+        *(uint32_t*)&hbuf[rt * 16 + c][16 * wave + 4 * rg] = word;
+        if (rg == 0 && (wave & 1) == 0) hes[rt * 16 + c][wave >> 1] = (unsigned char)e;
+    }
+    __syncthreads();
+    if (tid < 256) {
+        const int row = tid >> 3, ch = tid & 7;
+        if (row < it.n) *(uint4*)(hq + (int64_t)(it.off + row) * I + f0 + ch * 16) = *(const uint4*)&hbuf[row][ch * 16];
+    } else if (tid < 256 + GT_ROWS) {
+        const int row = tid - 256;
+        if (row < it.n) *(uint32_t*)(hs + (int64_t)(it.off + row) * (I >> 5) + (f0 >> 5)) = *(const uint32_t*)hes[row];
+    }
+}
+
+__global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __restrict__ hq, const uint8_t* __restrict__ hs, WMat w2, int H, int I,
+                                                           const int* __restrict__ G, const Item* __restrict__ items, float* __restrict__ out)
+{
+    __shared__ __align__(16) unsigned char xl[2][GT_ROWS * GT_XS];
+    __shared__ __align__(16) unsigned char xsl[2][GT_ROWS * 16];
+    if ((int)blockIdx.y >= *G) return;
+    const Item it = items[blockIdx.y];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, rg = lane >> 4;
+    const int n0 = blockIdx.x * GT_FEAT;
+    const int nkg = I >> 9;
+    const int nrt = (it.n + 15) >> 4;
+    const int64_t tile = ((int64_t)it.e * H + n0 + 16 * wave) >> 4;
+    const uint8_t* r2 = w2.w + tile * nkg * REC;
+    v4i a[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) a[s] = ld_a_step(r2, s, lane);
+    uint32_t sa = ld_a_scales(r2, lane);
+    const int srow = tid >> 4, sch = tid & 15;
+    const uint8_t* xrow = hq + (int64_t)(it.off + min(srow, it.n - 1)) * I + sch * 32;
+    const uint8_t* xsrow = hs + (int64_t)(it.off + min(tid & (GT_ROWS - 1), it.n - 1)) * (I >> 5);
+    unsigned char* const xdst = &xl[0][srow * GT_XS + sch * 32];
+    uint4 x0 = *(const uint4*)xrow, x1 = *(const uint4*)(xrow + 16), xsc = *(const uint4*)xsrow;
+    *(uint4*)xdst = x0; *(uint4*)(xdst + 16) = x1;
+    if (tid < GT_ROWS) *(uint4*)&xsl[0][tid * 16] = xsc;
+    {
+        const int k1 = min(1, nkg - 1);
+        x0 = *(const uint4*)(xrow + k1 * 512); x1 = *(const uint4*)(xrow + k1 * 512 + 16); xsc = *(const uint4*)(xsrow + k1 * 16);
+    }
+    __syncthreads();
+    v4f tot[2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) tot[rt] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int kg = 0; kg < nkg; ++kg) {
+        const int buf = kg & 1, kn = min(kg + 1, nkg - 1);
+        const uint8_t* n2 = r2 + (int64_t)kn * REC;
+        const uint32_t san = ld_a_scales(n2, lane);
+        v4f cur[2];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) { cur[rt] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(cur[rt])); }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                if (rt < nrt) {
+                    const unsigned char* bp = &xl[buf][(rt * 16 + c) * GT_XS + s * 128 + 16 * rg];
+                    const uint4 lo = *(const uint4*)bp, hi = *(const uint4*)(bp + 64);
+                    const v8i b = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+                    const uint32_t sb = *(const uint32_t*)&xsl[buf][(rt * 16 + c) * 16 + s * 4] >> (8 * rg);
+                    cur[rt] = mfma_group_step(s, a[s], b, cur[rt], sa, sb);
+                }
+            }
+            a[s] = ld_a_step(n2, s, lane);
+        }
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) tot[rt] += cur[rt];
+        sa = san;
+        unsigned char* d = xdst + (buf ^ 1) * (GT_ROWS * GT_XS);
+        *(uint4*)d = x0; *(uint4*)(d + 16) = x1;
+        if (tid < GT_ROWS) *(uint4*)&xsl[buf ^ 1][tid * 16] = xsc;
+        const int k2 = min(kg + 2, nkg - 1);
+        x0 = *(const uint4*)(xrow + k2 * 512); x1 = *(const uint4*)(xrow + k2 * 512 + 16); xsc = *(const uint4*)(xsrow + k2 * 16);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        const int row = rt * 16 + c;
+        if (row < it.n) *(float4*)(out + (int64_t)(it.off + row) * H + n0 + 16 * wave + 4 * rg) = make_float4(tot[rt][0], tot[rt][1], tot[rt][2], tot[rt][3]);
+    }
+}
+
 // y[r] = (add[r] + sum of the shared experts' outputs) + (sum_k routed out[pairmap[r, k]], k ascending)
 // reference ds41_mx.cu:302-317
 __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ out, const int* __restrict__ pairmap, const float* __restrict__ add,
@@ -284,11 +666,17 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
 // ---------------------------------------------------------------- host side
 // rows per item: 16 for decode sizes, up to 512 rows of an expert beyond (one pass over the expert's weights per item, which
 // stay in registers while the item's rows go by)
-inline int gr_of(int R) { return R <= 16 ? 16 : 512; }
-inline int gmax_of(int R, int TT, int ET)
+// rows per item: 16 for decode sizes; beyond, 32 for the grouped GEMM (T16 records, K a multiple of 512 that fits the decode
+// kernels' one-K-group-per-wave order) and up to 512 for the other layouts (one pass over the expert's weights per item)
+inline int gr_of(int R, bool gemm) { return R <= 16 ? 16 : gemm ? GT_ROWS : 512; }
+inline bool gemm_ok(int layout, int R, int H, int I)
+{
+    return layout == L_T16 && R > 16 && H % 512 == 0 && I % 512 == 0 && H / 512 <= UP_WAVES && I / 512 <= DN_WAVES && I % GT_FEAT == 0 && H % GT_FEAT == 0;
+}
+inline int gmax_of(int R, int TT, int ET, bool gemm)
 {
     const int64_t P = (int64_t)R * TT;
-    return (int)((P < ET ? P : ET) + P / gr_of(R) + 1);
+    return (int)((P < ET ? P : ET) + P / gr_of(R, gemm) + 1);
 }
 struct WsLayout {
     size_t G, items, pairmap, prow, pw, hq, hs, out, total;
@@ -299,7 +687,7 @@ inline WsLayout ws_layout(int R, int H, int I, int TT, int ET)
     WsLayout l;
     size_t o = 0;
     l.G = o; o += align256(16 + 64 * 4);                       // G + a few counters
-    l.items = o; o += align256(sizeof(Item) * (size_t)gmax_of(R, TT, ET));
+    l.items = o; o += align256(sizeof(Item) * (size_t)gmax_of(R, TT, ET, true));     // the finer of the two item sizes
     l.pairmap = o; o += align256(4 * P);
     l.prow = o; o += align256(4 * P);
     l.pw = o; o += align256(4 * P);
@@ -315,7 +703,8 @@ int moe_launch(const uint8_t* xq, const uint8_t* xs, int R, const int64_t* idx, 
                const uint8_t* s3, const uint8_t* w2, const uint8_t* s2, int H, int I, int topk, int E, int n_shared, const float* add, float* y, void* ws,
                int skip_combine, hipStream_t st)
 {
-    const int TT = topk + n_shared, ET = E + n_shared, GR = gr_of(R), Gm = gmax_of(R, TT, ET);
+    const bool gemm = gemm_ok(LAYOUT, R, H, I);
+    const int TT = topk + n_shared, ET = E + n_shared, GR = gr_of(R, gemm), Gm = gmax_of(R, TT, ET, gemm);
     const WsLayout l = ws_layout(R, H, I, TT, ET);
     char* base = (char*)ws;
     int* G = (int*)(base + l.G);
@@ -328,8 +717,15 @@ int moe_launch(const uint8_t* xq, const uint8_t* xs, int R, const int64_t* idx, 
     float* out = (float*)(base + l.out);
     group_kernel<<<1, 1024, 0, st>>>(idx, rw, R, topk, n_shared, E, GR, G, items, pairmap, prow, pw, G + 4, 64);
     const WMat m1{w1, s1, I, H, (int64_t)ET * I / 8}, m3{w3, s3, I, H, (int64_t)ET * I / 8}, m2{w2, s2, H, I, (int64_t)ET * H / 8};
-    up_kernel<LAYOUT><<<dim3(I / 32, Gm), 64 * UP_WAVES, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
-    down_kernel<LAYOUT><<<dim3(H / 32, Gm), 64 * DN_WAVES, 0, st>>>(hq, hs, m2, H, I, G, items, out);
+    if (gemm) {
+        up_gemm_kernel<<<dim3(I / GT_FEAT, Gm), 512, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
+        down_gemm_kernel<<<dim3(H / GT_FEAT, Gm), 512, 0, st>>>(hq, hs, m2, H, I, G, items, out);
+    } else {
+    if (((H >> 7) + 3) >> 2 <= UP_WAVES) up_res_kernel<LAYOUT><<<dim3(I / 32, Gm), 64 * UP_WAVES, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
+    else up_kernel<LAYOUT><<<dim3(I / 32, Gm), 64 * UP_WAVES, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
+    if (((I >> 7) + 3) >> 2 <= DN_WAVES) down_res_kernel<LAYOUT><<<dim3(H / 32, Gm), 64 * DN_WAVES, 0, st>>>(hq, hs, m2, H, I, G, items, out);
+    else down_kernel<LAYOUT><<<dim3(H / 32, Gm), 64 * DN_WAVES, 0, st>>>(hq, hs, m2, H, I, G, items, out);
+    }
     if (!skip_combine) {
         const int64_t n4 = (int64_t)R * (H / 4);
         combine_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(out, pairmap, add, y, R, H, topk, n_shared);
@@ -344,6 +740,11 @@ inline bool shapes_ok(int R, int H, int I, int topk, int E, int n_shared)
 
 int g_s2 = 0;          // scale blobs handed to the ds41_moe_mx* symbols are 2-bit coded (reference ds41_mx.cu:1304)
 
+#ifdef SPK_MX_TRACE
+}  // namespace
+extern "C" __attribute__((visibility("default"))) void spark_debug_mx_gemm_trace(long long* buf) { (void)hipMemcpyToSymbol(HIP_SYMBOL(g_gtrace), &buf, sizeof(buf)); }
+namespace {
+#endif
 }  // namespace
 
 // ================================================================ C ABI: runtime-sized entry points (no reference counterpart symbol)

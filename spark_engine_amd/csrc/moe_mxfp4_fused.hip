@@ -12,6 +12,11 @@
 //       outputs over inside the XCD; for every token row the block of the row's last item in launch order adds
 //       them up: (add + shared experts) + (routed experts in slot order), the reference's order.
 //
+// Block order.  Work is laid out in groups of GS blocks: block i of group g first does stage-1 unit i of item g, then
+// stage-2 unit i of item g - 1 (group 0 has no stage 2, the last group no stage 1).  A block issues its stage-2 weight loads
+// the moment its stage-1 registers are free, so the weight stream never pauses for a block to retire and another to start,
+// and the last item's stage-2 blocks hold their weights long before its h arrives.
+//
 // Exchange without counters: every exchanged 32-bit word of the workspace is EMPTY (all ones) between uses; a producer
 // stores its value (an all-ones value is altered to another NaN pattern), the single consumer of the word polls until it
 // is not EMPTY and stores EMPTY back.  h crosses XCDs (device-coherent stores and loads), the per-pair outputs stay in
@@ -33,6 +38,13 @@ constexpr uint32_t EMPTY = 0xffffffffu;
 constexpr uint64_t EMPTY2 = ~0ull;
 constexpr int RED_BYTES = NW * 4 * 4 * 64 * 4;
 
+long long* g_trace = nullptr;
+#ifdef SPK_MX_TRACE
+#define TRACE(i) do { if (a.trace && tid == 0) a.trace[(int64_t)bid * 16 + (i)] = wall_clock64(); } while (0)
+#else
+#define TRACE(i) do { } while (0)
+#endif
+
 struct MArgs {
     const void* x;                     // bf16 [R, H] (QUANT) or E4M3 [R, H]
     const uint8_t* xs;                 // UE8M0 [R, H / 32] (not QUANT)
@@ -43,7 +55,8 @@ struct MArgs {
     uint32_t* hsw;                     // [NBD][P][I / 32] its scales, one word each
     float* yd;                         // [P][H] per-pair outputs
     int* err;
-    int R, TT, topk, E, P, Gmax, H, I, NJ, NBD, nU;
+    long long* trace;                  // optional per-block time stamps (diagnostic builds), 16 per block
+    int R, TT, topk, E, P, Gmax, H, I, NJ, NBD, GS;        // GS = blocks per group (a multiple of 8)
 };
 
 __device__ __forceinline__ uint32_t ld_dev32(const void* p) { return __hip_atomic_load((const uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -106,7 +119,7 @@ template <int LAYOUT, bool QUANT, bool LOCAL>
 __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ int sidx[PMAXF], rows[RMAX], comb[RMAX], misc[4];
+    __shared__ int sidx[PMAXF], rowsU[RMAX], rowsD[RMAX], comb[RMAX], misc[4];
     __shared__ unsigned char isf[PMAXF];
     __shared__ float amx[NW][16];
     __shared__ __align__(16) uint32_t hbw[16][8];          // the block's 32 code bytes per item row
@@ -116,15 +129,26 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, rg = lane >> 4;
     const int bid = blockIdx.x;
-    const bool isU = bid < a.nU;
+    const int grpi = bid / a.GS, bi = bid % a.GS;          // GS % 8 == 0: column block bi runs on XCD bi % 8 in every group
     const int H = a.H, I = a.I;
-    if (isU) {
+    TRACE(0);
+    __builtin_amdgcn_s_setprio(2);
+    const bool hasU = grpi < a.Gmax && bi < a.NJ;
+    // both items of this block up front: the stage-2 loads must not wait for an index lookup later
+    Group gu{0, 0}, gd{0, 0};
+    if (hasU) gu = find_item(a, grpi, sidx, isf, rowsU, misc);
+    __syncthreads();
+    if (grpi >= 1 && bi < a.NBD) gd = find_item(a, grpi - 1, sidx, isf, rowsD, misc);
+    TRACE(1);
+    if (gu.n > 0) {
         // ================================================================ stage 1
-        __builtin_amdgcn_s_setprio(2);
-        const int g = bid / a.NJ, jb = bid % a.NJ, j0 = jb * 32;
-        const Group grp = find_item(a, g, sidx, isf, rows, misc);
-        if (grp.n == 0) return;
+        const Group grp = gu;
+        const int* rows = rowsU;
+        const int jb = bi, j0 = jb * 32;
         const int steps = H >> 7, nkg = (steps + 3) >> 2;
+        // route weight of this lane's item row, requested ahead of the weight rows
+        float wgt = 0.f;
+        if (c < grp.n) { const int pr = rows[c], k = pr % a.TT; wgt = k < a.topk ? a.rw[(int64_t)(pr / a.TT) * a.topk + k] : 1.0f; }
         // ---- the first K group of this wave's weight rows, then the activations of its K groups
         v4i A[4][4];
         uint32_t sa[4];
@@ -164,6 +188,7 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
                     }
                 }
         }
+        TRACE(2);
         const bool valid = c < grp.n;
         const int rc = valid ? c : 0;
         const int pair = rows[rc];
@@ -193,14 +218,14 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int v = 0; v < 4; ++v) red[wave][t][v][lane] = acc[t][v];
+        TRACE(3);
         __syncthreads();
+        TRACE(4);
         // epilogue: thread (wave = (tp, v), lane = (c, rg)) owns feature j0 + 16 tp + 4 rg + v of column c
         const int tp = wave >> 2, v = wave & 3;
         float gsum = 0.f, usum = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) { gsum += red[w][tp][v][lane]; usum += red[w][2 + tp][v][lane]; }
-        float wgt = 0.f;
-        if (valid) { const int k = pair % a.TT; wgt = k < a.topk ? a.rw[(int64_t)(pair / a.TT) * a.topk + k] : 1.0f; }
         const float gt = fminf(bf16_round(gsum), 10.f);
         const float up = fminf(fmaxf(bf16_round(usum), -10.f), 10.f);
         const float yv = bf16_round(silu(gt) * up * wgt);
@@ -226,18 +251,13 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
                 st_dev32(a.hc + row * (I >> 2) + jb * 8 + w, word);
             } else st_dev32(a.hsw + row * (I >> 5) + jb, he[cc]);
         }
-        return;
+        TRACE(5);
     }
     // ==================================================================== stage 2
-    int nb = -1, g = 0;
-    {
-        const int b = bid - a.nU, xcd = b % NXCD, li = b / NXCD;
-        const int q = (li / a.Gmax) * NXCD + xcd;          // column block q lives on XCD q % 8
-        if (q < a.NBD) { nb = q; g = li % a.Gmax; }
-    }
-    if (nb < 0) return;
-    const Group grp = find_item(a, g, sidx, isf, rows, misc);
-    if (grp.n == 0) return;
+    if (gd.n == 0) return;
+    const Group grp = gd;
+    const int* rows = rowsD;
+    const int nb = bi, g = grpi - 1;
     const int sub = wave >> 2, kw = wave & 3;              // 32-column half of the block, K group within a round
     const int n0 = nb * DC + sub * 32;
     const int steps = I >> 7, nkg = (steps + 3) >> 2;
@@ -248,6 +268,8 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
         load_group<LAYOUT>(a.w2, grp.e, n0, kg, lane, A[0], sa[0]);
         load_group<LAYOUT>(a.w2, grp.e, n0 + 16, kg, lane, A[1], sa[1]);
     }
+    TRACE(6);
+    __builtin_amdgcn_s_setprio(0);                         // waiting: the stage-1 waves of the CU's other block go first
     // token rows of this item that this block sums: those whose other experts all belong to earlier items
     if (a.R == 1) { if (tid == 0) comb[0] = g == a.P - 1; }
     else {
@@ -263,6 +285,10 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
     }
     if (tid == 0) misc[2] = 1;
     __syncthreads();
+    // the residual of the token row this wave sums later, requested ahead of the wait (a late request would queue behind
+    // the other blocks' weight rows)
+    float base = 0.f;
+    if (wave < grp.n && comb[wave] && a.add) base = a.add[(int64_t)(rows[wave] / a.TT) * H + nb * DC + lane];
     // B operands of a round in LDS: [kw][step][g4][row < n] x (8 code words + 1 scale word), written by the waves of half 0
     uint32_t* hl = (uint32_t*)extra;
     const bool valid = c < grp.n;
@@ -330,6 +356,7 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
             }
         }
         __syncthreads();
+        TRACE(7);
         if (rd == 0) __builtin_amdgcn_s_setprio(3);        // from here on this block is the critical path
         if (have && misc[2]) {
 #pragma unroll
@@ -344,6 +371,7 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
             }
         }
     }
+    TRACE(8);
     if (!misc[2]) { if (tid == 0) atomicExch(a.err, 1); return; }
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -364,10 +392,10 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
             if (LOCAL) *(uint32_t*)p = u; else st_dev32(p, u);
         }
     }
+    TRACE(9);
     // ---- the token rows this block sums: wave i takes item row i, lane = column
     if (wave < grp.n && comb[wave]) {
         const int tok = rows[wave] / a.TT, col = nb * DC + lane;
-        const float base = a.add ? a.add[(int64_t)tok * H + col] : 0.f;
         float* py[TTMAX];
 #pragma unroll
         for (int k = 0; k < TTMAX; ++k) py[k] = a.yd + (int64_t)(tok * a.TT + (k < a.TT ? k : 0)) * H + col;
@@ -397,6 +425,7 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
             a.y[(int64_t)tok * H + col] = accs + s;
         } else if (lane == 0) atomicExch(a.err, 1);
     }
+    TRACE(10);
 }
 
 __global__ void fill_kernel(uint32_t* p, int64_t n)
@@ -405,7 +434,7 @@ __global__ void fill_kernel(uint32_t* p, int64_t n)
     if (i < n) p[i] = i < HEAD / 4 ? 0u : EMPTY;
 }
 
-struct FPlan { int TT, ET, P, Gmax, NJ, NBD, nU, nD; size_t hc, hsw, yd, total, lds; };
+struct FPlan { int TT, ET, P, Gmax, NJ, NBD, GS, nblocks; size_t hc, hsw, yd, total, lds; };
 FPlan fplan(int R, int H, int I, int topk, int E, int n_shared)
 {
     FPlan p;
@@ -413,8 +442,8 @@ FPlan fplan(int R, int H, int I, int topk, int E, int n_shared)
     p.P = R * p.TT;
     p.Gmax = p.P < p.ET ? p.P : p.ET;
     p.NJ = I / 32; p.NBD = H / DC;
-    p.nU = p.Gmax * p.NJ;
-    p.nD = (p.NBD + NXCD - 1) / NXCD * NXCD * p.Gmax;
+    p.GS = ((p.NJ > p.NBD ? p.NJ : p.NBD) + NXCD - 1) / NXCD * NXCD;
+    p.nblocks = (p.Gmax + 1) * p.GS;
     size_t o = HEAD;
     auto take = [&](size_t n) { const size_t q = o; o += align256(n); return q; };
     p.hc = take((size_t)p.NBD * p.P * I);
@@ -435,7 +464,7 @@ __global__ void xcd_probe_kernel(int* out)
 template <int LAYOUT, bool QUANT>
 int launch(const MArgs& a, const FPlan& p, hipStream_t st)
 {
-    const dim3 grid(p.nU + p.nD), blk(NT);
+    const dim3 grid(p.nblocks), blk(NT);
     if (g_local == 1) {
         static bool attr = false;
         if (!attr) { (void)hipFuncSetAttribute((const void*)mx_fused_kernel<LAYOUT, QUANT, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); attr = true; }
@@ -499,7 +528,8 @@ int mx_fused_launch(const void* x, const void* xs, int R, const int64_t* idx, co
     a.w2 = WMat{(const uint8_t*)w2, (const uint8_t*)s2, H, I, ET * H / 8};
     a.add = add; a.y = y;
     a.hc = (uint32_t*)(b + p.hc); a.hsw = (uint32_t*)(b + p.hsw); a.yd = (float*)(b + p.yd); a.err = (int*)b;
-    a.R = R; a.TT = p.TT; a.topk = topk; a.E = E; a.P = p.P; a.Gmax = p.Gmax; a.H = H; a.I = I; a.NJ = p.NJ; a.NBD = p.NBD; a.nU = p.nU;
+    a.R = R; a.TT = p.TT; a.topk = topk; a.E = E; a.P = p.P; a.Gmax = p.Gmax; a.H = H; a.I = I; a.NJ = p.NJ; a.NBD = p.NBD; a.GS = p.GS;
+    a.trace = g_trace;
     if (!clean) {
         const int rc = mx_fused_ws_prepare(ws, p.total, st);
         if (rc) return rc;
@@ -513,6 +543,10 @@ int mx_fused_launch(const void* x, const void* xs, int R, const int64_t* idx, co
     }
     return 1;
 }
+
+// diagnostics: device buffer of 16 time stamps (100 MHz) per block of the next launches, or null (recorded by builds with
+// -DSPK_MX_TRACE only)
+extern "C" __attribute__((visibility("default"))) void spark_debug_mx_trace(long long* buf) { g_trace = buf; }
 
 }  // namespace mx
 }  // namespace spk
