@@ -103,25 +103,39 @@ __global__ void fp8_e8m0_dequant_kernel(const uint8_t* __restrict__ w, const uin
     out[i] = e4m3_to_f32(w[i]) * e8m0_to_f32(s[(int64_t)(n >> 5) * (K >> 5) + (k >> 5)]);
 }
 
-// ---------------------------------------------------------------- act_quant: 32 lanes per block of 32, two blocks per wave
+// ---------------------------------------------------------------- act_quant: 4 lanes x 8 elements per block of 32
 template <bool BYTES>
 __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ outb, uint8_t* __restrict__ q,
                                                         uint8_t* __restrict__ s, int64_t blocks)
 {
-    const int64_t b = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
-    const int l = threadIdx.x & 31;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t b = t >> 2;                          // lanes 4j .. 4j+3 of a wave share block b (blocks are whole or absent per quad)
     if (b >= blocks) return;
-    const float v = bf16_to_f32(x[b * 32 + l]);
-    float a = fabsf(v);
+    const uint4 raw = *(const uint4*)(x + t * 8);
+    const uint32_t rw4[4] = {raw.x, raw.y, raw.z, raw.w};
+    float v[8];
+    float a = 0.f;
 #pragma unroll
-    for (int o = 16; o; o >>= 1) a = fmaxf(a, __shfl_xor(a, o, 64));     // stays inside the half-wave
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(rw4[i] << 16); v[2 * i + 1] = __uint_as_float(rw4[i] & 0xffff0000u);
+        a = fmaxf(a, fmaxf(fabsf(v[2 * i]), fabsf(v[2 * i + 1])));
+    }
+    a = fmaxf(a, __shfl_xor(a, 1, 64));
+    a = fmaxf(a, __shfl_xor(a, 2, 64));
     const uint32_t e = aq_scale(a);
-    const uint32_t byte = aq_byte(v, e);
     if (BYTES) {
-        q[b * 32 + l] = (uint8_t)byte;
-        if (l == 0) s[b] = (uint8_t)e;
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { lo |= aq_byte(v[i], e) << (8 * i); hi |= aq_byte(v[4 + i], e) << (8 * i); }
+        *(uint2*)(q + t * 8) = make_uint2(lo, hi);
+        if ((t & 3) == 0) s[b] = (uint8_t)e;
     } else {
-        outb[b * 32 + l] = f32_to_bf16(e4m3_to_f32(byte) * __uint_as_float(e << 23));
+        uint32_t o[4];
+        const float sc = __uint_as_float(e << 23);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            o[i] = (uint32_t)f32_to_bf16(e4m3_to_f32(aq_byte(v[2 * i], e)) * sc) | ((uint32_t)f32_to_bf16(e4m3_to_f32(aq_byte(v[2 * i + 1], e)) * sc) << 16);
+        *(uint4*)(outb + t * 8) = make_uint4(o[0], o[1], o[2], o[3]);
     }
 }
 
@@ -224,7 +238,7 @@ SPARK_API int ds41_act_quant32(const void* x, void* out, long long numel, hipStr
     if (numel % 32) return 1;
     const long long blocks = numel / 32;
     if (blocks == 0) return 0;
-    act_quant_kernel<false><<<(unsigned)((blocks + 7) / 8), 256, 0, st>>>((const uint16_t*)x, (uint16_t*)out, nullptr, nullptr, blocks);
+    act_quant_kernel<false><<<(unsigned)((blocks + 63) / 64), 256, 0, st>>>((const uint16_t*)x, (uint16_t*)out, nullptr, nullptr, blocks);
     return launch_status();
 }
 // reference ds41_mx.cu:1394-1399
@@ -233,7 +247,7 @@ SPARK_API int ds41_act_quant_fp8(const void* x, void* q, void* s, long long nume
     if (numel % 32) return 1;
     const long long blocks = numel / 32;
     if (blocks == 0) return 0;
-    act_quant_kernel<true><<<(unsigned)((blocks + 7) / 8), 256, 0, st>>>((const uint16_t*)x, nullptr, (uint8_t*)q, (uint8_t*)s, blocks);
+    act_quant_kernel<true><<<(unsigned)((blocks + 63) / 64), 256, 0, st>>>((const uint16_t*)x, nullptr, (uint8_t*)q, (uint8_t*)s, blocks);
     return launch_status();
 }
 // reference ds41_ops.cu:615 (ds41_swiglu_quant)

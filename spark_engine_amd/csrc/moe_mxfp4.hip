@@ -53,10 +53,17 @@ __global__ __launch_bounds__(1024) void group_kernel(const int64_t* __restrict__
     for (int i = tid; i < ncounters; i += 1024) counters[i] = 0;
     for (int e = tid; e < ET; e += 1024) { cnt[e] = 0; fill[e] = 0; }
     __syncthreads();
-    for (int p = tid; p < P; p += 1024) {
-        const int r = p / TT, k = p % TT;
-        const int e = k < topk ? (int)idx[(int64_t)r * topk + k] : E + (k - topk);
-        atomicAdd(&cnt[e], 1);
+    // eight pairs per thread at a time: their index loads are in flight together (one workgroup has no other latency hiding)
+    for (int p0 = tid; p0 < P; p0 += 8 * 1024) {
+        int ev[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int p = min(p0 + u * 1024, P - 1), r = p / TT, k = p % TT;
+            ev[u] = k < topk ? (int)idx[(int64_t)r * topk + k] : E + (k - topk);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (p0 + u * 1024 < P) atomicAdd(&cnt[ev[u]], 1);
     }
     __syncthreads();
     // exclusive scans of rows and items over the experts (two experts per thread)
@@ -84,13 +91,25 @@ __global__ __launch_bounds__(1024) void group_kernel(const int64_t* __restrict__
         const int c = cnt[e];
         for (int j = 0; j * GR < c; ++j) items[ioff[e] + j] = Item{e, eoff[e] + j * GR, min(GR, c - j * GR), 0};
     }
-    for (int p = tid; p < P; p += 1024) {
-        const int r = p / TT, k = p % TT;
-        const int e = k < topk ? (int)idx[(int64_t)r * topk + k] : E + (k - topk);
-        const int pos = eoff[e] + atomicAdd(&fill[e], 1);
-        pairmap[p] = pos;
-        prow[pos] = p;
-        pw[pos] = k < topk ? rw[(int64_t)r * topk + k] : 1.0f;
+    for (int p0 = tid; p0 < P; p0 += 8 * 1024) {
+        int ev[8];
+        float wv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int p = min(p0 + u * 1024, P - 1), r = p / TT, k = p % TT;
+            ev[u] = k < topk ? (int)idx[(int64_t)r * topk + k] : E + (k - topk);
+            wv[u] = k < topk ? rw[(int64_t)r * topk + k] : 1.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int p = p0 + u * 1024;
+            if (p < P) {
+                const int pos = eoff[ev[u]] + atomicAdd(&fill[ev[u]], 1);
+                pairmap[p] = pos;
+                prow[pos] = p;
+                pw[pos] = wv[u];
+            }
+        }
     }
 }
 
@@ -413,10 +432,12 @@ constexpr int GT_FEAT = 128;           // output features / columns of a block
 
 __device__ __forceinline__ v4i ld_a_step(const uint8_t* rec, int s, int lane)
 {
-    const uint4 v = ld_stream16(rec + s * 1024 + lane * 16);
+    // default cache policy, not a streaming load: an expert's other 32-row items (neighbours in launch order, on the same XCD)
+    // read the same records and find them in the L2 (measured: 1.45 -> 1.25 ms on the 2048-token workload)
+    const uint4 v = *(const uint4*)(rec + s * 1024 + lane * 16);
     return v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
 }
-__device__ __forceinline__ uint32_t ld_a_scales(const uint8_t* rec, int lane) { return __builtin_nontemporal_load((const uint32_t*)(rec + 4096 + lane * 4)); }
+__device__ __forceinline__ uint32_t ld_a_scales(const uint8_t* rec, int lane) { return *(const uint32_t*)(rec + 4096 + lane * 4); }
 
 __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, WMat w1, WMat w3, int H, int I, int TT,
                                                          const int* __restrict__ G, const Item* __restrict__ items, const int* __restrict__ prow,
@@ -429,8 +450,8 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
     __shared__ float amx[8][2][16];
     __shared__ __align__(16) unsigned char hbuf[GT_ROWS][GT_FEAT + 16];
     __shared__ __align__(4) unsigned char hes[GT_ROWS][4];
+    const Item it = items[blockIdx.y];             // requested together with the item count (entries past it hold anything)
     if ((int)blockIdx.y >= *G) return;
-    const Item it = items[blockIdx.y];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, rg = lane >> 4;
     const int f0 = blockIdx.x * GT_FEAT;
     const int nkg = H >> 9;
@@ -544,23 +565,26 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
     }
 }
 
+constexpr int GT_COLS = 256;           // output columns of a down-projection block: two 16-column tiles per wave
 __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __restrict__ hq, const uint8_t* __restrict__ hs, WMat w2, int H, int I,
                                                            const int* __restrict__ G, const Item* __restrict__ items, float* __restrict__ out)
 {
     __shared__ __align__(16) unsigned char xl[2][GT_ROWS * GT_XS];
     __shared__ __align__(16) unsigned char xsl[2][GT_ROWS * 16];
+    const Item it = items[blockIdx.y];             // requested together with the item count (entries past it hold anything)
     if ((int)blockIdx.y >= *G) return;
-    const Item it = items[blockIdx.y];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, rg = lane >> 4;
-    const int n0 = blockIdx.x * GT_FEAT;
+    const int n0 = blockIdx.x * GT_COLS + 32 * wave;
     const int nkg = I >> 9;
     const int nrt = (it.n + 15) >> 4;
-    const int64_t tile = ((int64_t)it.e * H + n0 + 16 * wave) >> 4;
-    const uint8_t* r2 = w2.w + tile * nkg * REC;
-    v4i a[4];
+    const int64_t tile = ((int64_t)it.e * H + n0) >> 4;
+    const uint8_t* ra = w2.w + tile * nkg * REC;
+    const uint8_t* rb = ra + (int64_t)nkg * REC;
+    v4i a[2][4];
+    uint32_t sa[2];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) a[s] = ld_a_step(r2, s, lane);
-    uint32_t sa = ld_a_scales(r2, lane);
+    for (int s = 0; s < 4; ++s) { a[0][s] = ld_a_step(ra, s, lane); a[1][s] = ld_a_step(rb, s, lane); }
+    sa[0] = ld_a_scales(ra, lane); sa[1] = ld_a_scales(rb, lane);
     const int srow = tid >> 4, sch = tid & 15;
     const uint8_t* xrow = hq + (int64_t)(it.off + min(srow, it.n - 1)) * I + sch * 32;
     const uint8_t* xsrow = hs + (int64_t)(it.off + min(tid & (GT_ROWS - 1), it.n - 1)) * (I >> 5);
@@ -573,16 +597,21 @@ __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __rest
         x0 = *(const uint4*)(xrow + k1 * 512); x1 = *(const uint4*)(xrow + k1 * 512 + 16); xsc = *(const uint4*)(xsrow + k1 * 16);
     }
     __syncthreads();
-    v4f tot[2];
+    v4f tot[2][2];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) tot[rt] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) tot[m][rt] = v4f{0.f, 0.f, 0.f, 0.f};
     for (int kg = 0; kg < nkg; ++kg) {
         const int buf = kg & 1, kn = min(kg + 1, nkg - 1);
-        const uint8_t* n2 = r2 + (int64_t)kn * REC;
-        const uint32_t san = ld_a_scales(n2, lane);
-        v4f cur[2];
+        const uint8_t* na = ra + (int64_t)kn * REC;
+        const uint8_t* nb = rb + (int64_t)kn * REC;
+        const uint32_t san0 = ld_a_scales(na, lane), san1 = ld_a_scales(nb, lane);
+        v4f cur[2][2];
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) { cur[rt] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(cur[rt])); }
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) { cur[m][rt] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(cur[m][rt])); }
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
 #pragma unroll
@@ -592,14 +621,18 @@ __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __rest
                     const uint4 lo = *(const uint4*)bp, hi = *(const uint4*)(bp + 64);
                     const v8i b = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
                     const uint32_t sb = *(const uint32_t*)&xsl[buf][(rt * 16 + c) * 16 + s * 4] >> (8 * rg);
-                    cur[rt] = mfma_group_step(s, a[s], b, cur[rt], sa, sb);
+                    cur[0][rt] = mfma_group_step(s, a[0][s], b, cur[0][rt], sa[0], sb);
+                    cur[1][rt] = mfma_group_step(s, a[1][s], b, cur[1][rt], sa[1], sb);
                 }
             }
-            a[s] = ld_a_step(n2, s, lane);
+            a[0][s] = ld_a_step(na, s, lane);
+            a[1][s] = ld_a_step(nb, s, lane);
         }
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) tot[rt] += cur[rt];
-        sa = san;
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) tot[m][rt] += cur[m][rt];
+        sa[0] = san0; sa[1] = san1;
         unsigned char* d = xdst + (buf ^ 1) * (GT_ROWS * GT_XS);
         *(uint4*)d = x0; *(uint4*)(d + 16) = x1;
         if (tid < GT_ROWS) *(uint4*)&xsl[buf ^ 1][tid * 16] = xsc;
@@ -610,7 +643,11 @@ __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __rest
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
         const int row = rt * 16 + c;
-        if (row < it.n) *(float4*)(out + (int64_t)(it.off + row) * H + n0 + 16 * wave + 4 * rg) = make_float4(tot[rt][0], tot[rt][1], tot[rt][2], tot[rt][3]);
+        if (row < it.n) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+                *(float4*)(out + (int64_t)(it.off + row) * H + n0 + 16 * m + 4 * rg) = make_float4(tot[m][rt][0], tot[m][rt][1], tot[m][rt][2], tot[m][rt][3]);
+        }
     }
 }
 
@@ -671,7 +708,7 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
 inline int gr_of(int R, bool gemm) { return R <= 16 ? 16 : gemm ? GT_ROWS : 512; }
 inline bool gemm_ok(int layout, int R, int H, int I)
 {
-    return layout == L_T16 && R > 16 && H % 512 == 0 && I % 512 == 0 && H / 512 <= UP_WAVES && I / 512 <= DN_WAVES && I % GT_FEAT == 0 && H % GT_FEAT == 0;
+    return layout == L_T16 && R > 16 && H % 512 == 0 && I % 512 == 0 && H / 512 <= UP_WAVES && I / 512 <= DN_WAVES && I % GT_FEAT == 0 && H % GT_COLS == 0;
 }
 inline int gmax_of(int R, int TT, int ET, bool gemm)
 {
@@ -719,7 +756,7 @@ int moe_launch(const uint8_t* xq, const uint8_t* xs, int R, const int64_t* idx, 
     const WMat m1{w1, s1, I, H, (int64_t)ET * I / 8}, m3{w3, s3, I, H, (int64_t)ET * I / 8}, m2{w2, s2, H, I, (int64_t)ET * H / 8};
     if (gemm) {
         up_gemm_kernel<<<dim3(I / GT_FEAT, Gm), 512, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
-        down_gemm_kernel<<<dim3(H / GT_FEAT, Gm), 512, 0, st>>>(hq, hs, m2, H, I, G, items, out);
+        down_gemm_kernel<<<dim3(H / GT_COLS, Gm), 512, 0, st>>>(hq, hs, m2, H, I, G, items, out);
     } else {
     if (((H >> 7) + 3) >> 2 <= UP_WAVES) up_res_kernel<LAYOUT><<<dim3(I / 32, Gm), 64 * UP_WAVES, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
     else up_kernel<LAYOUT><<<dim3(I / 32, Gm), 64 * UP_WAVES, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
