@@ -178,6 +178,8 @@ SPARK_API int ds41_moe(const void* xq, int R, const int64_t* idx, const float* r
  * flags bit 1: force the several-kernel path.
  * flags bit 2: tab has a tenth row, uint64 [E], with each expert's trellis width (3..6 bits, engine-rs/shim/moe_exl3.cuh:239-252); all
  * three matrices of an expert share it.  Runs on the several-kernel path.
+ * flags bit 3: tab has an eleventh row with each expert's own intermediate width (a multiple of 128, at most I; I is then the stride
+ * of the intermediates); gate / up have that many columns, down that many rows.  Runs on the several-kernel path.
  * Replaces engine-rs/shim/moe_exl3.cuh:1512-1691 (moex::experts). */
 SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk);
 SPARK_API int spark_exl3_moe_ws_init(void* ws, size_t bytes, hipStream_t st);
@@ -194,6 +196,13 @@ SPARK_API int qwen_moe_experts(const void* x, int64_t ldx, int R, const void* id
 SPARK_API size_t glm_moe_ws_bytes(int R, int S);
 SPARK_API int glm_moe_experts(const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out,
                               void* ws, int S, const void* suh0, int kmask, hipStream_t st);
+/* GLM under a three-way split of every expert: each expert 768 or 640 wide (6 or 5 of its 128-wide Hadamard blocks).  tab = uint64
+ * [11][288]: rows 0-8 as above, row 9 the trellis width in bits (read when kmask is not 1 << 4), row 10 the expert's intermediate
+ * width; gate / up trellis [H/16, width/16, 16 bits] int16, down [width/16, H/16, 16 bits].  Everything else as glm_moe_experts.
+ * Replaces engine-rs/shim/glm_moe.cu:17-24 (moex::GlmMoe3, engine-rs/shim/moe_exl3.cuh:63-67,132-136). */
+SPARK_API size_t glm_moe3_ws_bytes(int R, int S);
+SPARK_API int glm_moe3_experts(const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out,
+                               void* ws, int S, int kmask, hipStream_t st);
 
 /* ---------------------------------------------------------------- diagnostics (not part of the reference ABI) ---------------- */
 

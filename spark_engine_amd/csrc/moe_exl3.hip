@@ -108,18 +108,22 @@ template <int CBK, int MR>
 __global__ __launch_bounds__(64 * GV_WAVES) void gemv_kernel(const uint16_t* __restrict__ xh, const uint64_t* __restrict__ tab, int E, int tr_slot0,
                                                              const int* __restrict__ G, const int* __restrict__ gexp, const int* __restrict__ goff,
                                                              const int* __restrict__ gcnt, int Gmax, int T, int P, int K, int N, int kts,
-                                                             float* __restrict__ part)
+                                                             float* __restrict__ part, int vw)
 {
     __shared__ float red[GV_WAVES][MR][128];
     const int tg = blockIdx.z, t = tg / Gmax, g = tg % Gmax;
     if (g >= *G) return;
     const int rows = gcnt[g];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int Nt = N / 16, nb = blockIdx.x, s = blockIdx.y;
+    // vw: the expert's own intermediate width (row 10 of the table) replaces N (1: gate / up) or K (2: down); strides keep N / K
+    const int we = vw ? (int)tab[(int64_t)10 * E + gexp[g]] : 0;
+    const int Ne = vw == 1 ? we : N, Ke = vw == 2 ? we : K;
+    const int Nt = Ne / 16, nb = blockIdx.x, s = blockIdx.y;
+    if (nb * 128 >= Ne) return;
     const uint32_t* tr = (const uint32_t*)tab[(int64_t)(tr_slot0 + t) * E + gexp[g]];
     const int64_t r0 = (int64_t)t * P + goff[g];
     const uint32_t* xbase = (const uint32_t*)(xh + r0 * K);   // rows K fp16 = K/2 words apart
-    const int kt0 = s * kts, kt1 = min(K / 16, kt0 + kts);
+    const int kt0 = s * kts, kt1 = min(Ke / 16, kt0 + kts);
     float acc[MR][2];
 #pragma unroll
     for (int r = 0; r < MR; ++r) { acc[r][0] = 0.f; acc[r][1] = 0.f; }
@@ -154,7 +158,7 @@ template <int CBK>
 __global__ __launch_bounds__(256) void gemv_anybits_kernel(const uint16_t* __restrict__ xh, const uint64_t* __restrict__ tab, int E, int tr_slot0,
                                                           const int* __restrict__ G, const int* __restrict__ gexp, const int* __restrict__ goff,
                                                           const int* __restrict__ gcnt, int Gmax, int T, int P, int K, int N, int kts,
-                                                          float* __restrict__ part)
+                                                          float* __restrict__ part, int vw)
 {
     __shared__ uint16_t wl[16 * 128];
     __shared__ uint32_t tw[8 * 48];
@@ -163,11 +167,14 @@ __global__ __launch_bounds__(256) void gemv_anybits_kernel(const uint16_t* __res
     const int rows = gcnt[g], e = gexp[g];
     const int bits = (int)tab[(int64_t)9 * E + e], nw = 8 * bits;
     const int tid = threadIdx.x, col = tid & 127, half = tid >> 7;
-    const int Nt = N / 16, nb = blockIdx.x, s = blockIdx.y;
+    const int we = vw ? (int)tab[(int64_t)10 * E + e] : 0;
+    const int Ne = vw == 1 ? we : N, Ke = vw == 2 ? we : K;
+    const int Nt = Ne / 16, nb = blockIdx.x, s = blockIdx.y;
+    if (nb * 128 >= Ne) return;
     const uint32_t* tr = (const uint32_t*)tab[(int64_t)(tr_slot0 + t) * E + e];
     const int64_t r0 = (int64_t)t * P + goff[g];
     const uint16_t* xbase = xh + r0 * K;
-    const int kt0 = s * kts, kt1 = min(K / 16, kt0 + kts);
+    const int kt0 = s * kts, kt1 = min(Ke / 16, kt0 + kts);
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
@@ -211,12 +218,13 @@ __global__ __launch_bounds__(256) void gemv_anybits_kernel(const uint16_t* __res
 // ---------------------------------------------------------------- mid: finish gate and up, act, down input transform
 // wave per (compact row, 128-block of I); reference moe_exl3.cuh:1019-1064
 __global__ __launch_bounds__(256) void mid_kernel(const float* __restrict__ part, int S, const uint64_t* __restrict__ tab, int E, int P, int I, int act,
-                                                  const int* __restrict__ pexp, uint16_t* __restrict__ xh2)
+                                                  const int* __restrict__ pexp, uint16_t* __restrict__ xh2, int vw)
 {
     const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, lane = threadIdx.x & 63;
     const int nb = I / 128, b = wave % nb, row = wave / nb;
     if (row >= P) return;
     const int e = pexp[row], n = b * 128 + 2 * lane;
+    if (vw && b * 128 >= (int)tab[(int64_t)10 * E + e]) return;      // past the expert's own width: the down product never reads it
     float g[2][2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -299,30 +307,32 @@ inline bool cfg_ok(const Cfg& c, int R)
 
 template <int CBK>
 void launch_gemv(const uint16_t* xh, const uint64_t* tab, int E, int slot0, const int* G, const int* gexp, const int* goff, const int* gcnt, int Gmax, int T,
-                 int P, int K, int N, int S, int maxrows, float* part, hipStream_t st, bool mixed = false)
+                 int P, int K, int N, int S, int maxrows, float* part, hipStream_t st, bool mixed, int vw)
 {
     const dim3 grid(N / 128, S, T * Gmax), blk(64 * GV_WAVES);
     const int kts = (K / 16 + S - 1) / S;
     if (mixed) {                                     // per-expert trellis widths from row 9 of the table
-        gemv_anybits_kernel<CBK><<<grid, 256, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
+        gemv_anybits_kernel<CBK><<<grid, 256, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part, vw);
         return;
     }
     // one instantiation per row-count class of the call (items never hold more rows than the call has)
-    if (maxrows <= 1) gemv_kernel<CBK, 1><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
-    else if (maxrows <= 2) gemv_kernel<CBK, 2><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
-    else if (maxrows <= 4) gemv_kernel<CBK, 4><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
-    else if (maxrows <= 8) gemv_kernel<CBK, 8><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
-    else gemv_kernel<CBK, 16><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part);
+    if (maxrows <= 1) gemv_kernel<CBK, 1><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part, vw);
+    else if (maxrows <= 2) gemv_kernel<CBK, 2><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part, vw);
+    else if (maxrows <= 4) gemv_kernel<CBK, 4><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part, vw);
+    else if (maxrows <= 8) gemv_kernel<CBK, 8><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part, vw);
+    else gemv_kernel<CBK, 16><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part, vw);
 }
 
 // flags: bit 0 = the workspace is prepared (once, then only used by these calls);
-//        bit 1 = force the multi-kernel path; bit 2 = mixed trellis widths (table row 9 = bits per expert; multi-kernel path)
+//        bit 1 = force the multi-kernel path; bit 2 = mixed trellis widths (table row 9 = bits per expert; multi-kernel path);
+//        bit 3 = every expert has its own intermediate width (table row 10, a multiple of 128 up to I; multi-kernel path)
 int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
             int flags, hipStream_t st)
 {
     if (!cfg_ok(c, R)) return -1;
     const bool mixed = (flags & 4) != 0;             // the table has a row 9 with every expert's trellis width (3..6 bits)
-    if (!(flags & 2) && !mixed && exl3_fused_ok(c, R)) return exl3_fused_launch(c, x, ldx, R, idx, w, tab, add, out, ws, flags & 1, st);
+    const bool varw = (flags & 8) != 0;              // and a row 10 with every expert's intermediate width (reference moe_exl3.cuh:63-67,132-136)
+    if (!(flags & 2) && !mixed && !varw && exl3_fused_ok(c, R)) return exl3_fused_launch(c, x, ldx, R, idx, w, tab, add, out, ws, flags & 1, st);
     const Plan p = plan(c, R);
     char* b = (char*)ws + (exl3_fused_ok(c, R) ? exl3_fused_ws_bytes(c, R) : 0);       // the two paths never share workspace bytes
     int* G = (int*)(b + p.G);
@@ -336,12 +346,12 @@ int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, co
     prep_kernel<<<1, EMAX, 0, st>>>(idx, c.itype, R, c.topk, c.E, GR, G, gexp, goff, gcnt, pairmap, prow, pexp);
     int waves = 2 * p.P * (c.H / 128);
     had_kernel<<<(waves + 3) / 4, 256, 0, st>>>(x, c.xtype, ldx, tb, c.E, 3, 2, p.P, prow, pexp, c.H, xh1);
-    if (c.cbk == CB_MCG) launch_gemv<CB_MCG>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, p.S1, maxrows, part, st, mixed);
-    else launch_gemv<CB_MUL1>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, p.S1, maxrows, part, st, mixed);
+    if (c.cbk == CB_MCG) launch_gemv<CB_MCG>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, p.S1, maxrows, part, st, mixed, varw ? 1 : 0);
+    else launch_gemv<CB_MUL1>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, p.S1, maxrows, part, st, mixed, varw ? 1 : 0);
     waves = p.P * (c.I / 128);
-    mid_kernel<<<(waves + 3) / 4, 256, 0, st>>>(part, p.S1, tb, c.E, p.P, c.I, c.act, pexp, xh2);
-    if (c.cbk == CB_MCG) launch_gemv<CB_MCG>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, p.S2, maxrows, part, st, mixed);
-    else launch_gemv<CB_MUL1>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, p.S2, maxrows, part, st, mixed);
+    mid_kernel<<<(waves + 3) / 4, 256, 0, st>>>(part, p.S1, tb, c.E, p.P, c.I, c.act, pexp, xh2, varw ? 1 : 0);
+    if (c.cbk == CB_MCG) launch_gemv<CB_MCG>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, p.S2, maxrows, part, st, mixed, varw ? 2 : 0);
+    else launch_gemv<CB_MUL1>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, p.S2, maxrows, part, st, mixed, varw ? 2 : 0);
     waves = R * (c.H / 128);
     finish_combine_kernel<<<(waves + 3) / 4, 256, 0, st>>>(part, p.S2, tb, c.E, p.P, c.H, c.topk, pairmap, pexp, w, c.wtype, (const float*)add, (float*)out, R);
     return launch_status();
@@ -349,6 +359,7 @@ int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, co
 
 const Cfg QWEN{512, 10, 2560, 640, CB_MUL1, 0, X_F32, 0, 0};
 const Cfg GLM{288, 8, 4096, 1024, CB_MCG, 1, X_F16, 1, 1};
+const Cfg GLM3{288, 8, 4096, 768, CB_MCG, 1, X_F16, 1, 1};        // TP3: experts 640 or 768 wide, I = the widest (strides)
 
 }  // namespace
 
@@ -397,4 +408,15 @@ SPARK_API int glm_moe_experts(const void* x, int64_t ldx, int R, const void* idx
     (void)S; (void)suh0;
     if (kmask <= 0 || (kmask & ~0x78)) return -4;              // widths 3..6 only
     return experts(GLM, x, ldx, R, idx, w, tab, add, out, ws, kmask == (1 << 4) ? 0 : 4, st);
+}
+// reference glm_moe.cu:17-24 (moex::GlmMoe3, moe_exl3.cuh:63-67): GLM under a three-way split, every expert 768 or 640 wide (6 or
+// 5 of its 128-wide Hadamard blocks); tab u64 [11][288]: rows 0-8 as above, row 9 the trellis width in bits, row 10 the
+// expert's intermediate width.  Intermediates keep the stride of the widest expert (768).
+SPARK_API size_t glm_moe3_ws_bytes(int R, int S) { (void)S; return spark_exl3_moe_ws_bytes(R, GLM3.H, GLM3.I, GLM3.E, GLM3.topk); }
+SPARK_API int glm_moe3_experts(const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws, int S,
+                               int kmask, hipStream_t st)
+{
+    (void)S;
+    if (kmask <= 0 || (kmask & ~0x78)) return -4;
+    return experts(GLM3, x, ldx, R, idx, w, tab, add, out, ws, 8 | (kmask == (1 << 4) ? 0 : 4), st);
 }

@@ -75,6 +75,8 @@ SIGNATURES = {
     "qwen_moe_experts": (i32, [vp, i64, i32, vp, vp, vp, vp, vp, vp, i32, vp]),
     "glm_moe_ws_bytes": (sz, [i32, i32]),
     "glm_moe_experts": (i32, [vp, i64, i32, vp, vp, vp, vp, vp, vp, i32, vp, i32, vp]),
+    "glm_moe3_ws_bytes": (sz, [i32, i32]),
+    "glm_moe3_experts": (i32, [vp, i64, i32, vp, vp, vp, vp, vp, vp, i32, i32, vp]),
 }
 
 _lib = None

@@ -406,19 +406,24 @@ class ExpertTable:
     """All experts of one layer resident on the GPU + the [9][E] device-pointer table (gate_tr, up_tr, down_tr,
     gate_suh, up_suh, down_suh, gate_svh, up_svh, down_svh)."""
 
-    def __init__(self, experts, E, device="cuda:0", bits=None):
+    def __init__(self, experts, E, device="cuda:0", bits=None, widths=None):
         """experts: dict e -> 9 device tensors (or stacked tensors per slot, see from_stacked).  Missing experts get null pointers.
-        bits: dict e -> trellis width of the expert (3..6): adds row 9 of the reference's mixed-width tables (moe_exl3.cuh:239-252)."""
+        bits: dict e -> trellis width of the expert (3..6): adds row 9 of the reference's mixed-width tables (moe_exl3.cuh:239-252).
+        widths: dict e -> intermediate width of the expert: adds row 10 (and row 9, 4 bits unless bits is given) of the reference's
+        variable-width tables (moe_exl3.cuh:63-67,132-136)."""
         self.E = E
         self.keep = experts
-        rows = [[0] * E for _ in range(9 if bits is None else 10)]
+        rows = [[0] * E for _ in range(11 if widths is not None else 9 if bits is None else 10)]
         for e, ts in experts.items():
             for slot, t in enumerate(ts):
                 assert t.is_cuda and t.is_contiguous()
                 rows[slot][e] = t.data_ptr()
-            if bits is not None:
-                rows[9][e] = int(bits[e])
+            if bits is not None or widths is not None:
+                rows[9][e] = int(bits[e]) if bits is not None else 4
+            if widths is not None:
+                rows[10][e] = int(widths[e])
         self.mixed = bits is not None
+        self.varw = widths is not None
         self.kmask = 1 << 4 if bits is None else sum({1 << int(b) for b in bits.values()})
         self.tab = torch.tensor(rows, dtype=torch.int64, device=device).contiguous()
 
@@ -454,7 +459,7 @@ def exl3_moe(x, idx, w, table, H, I, codebook=2, act=0, add=None, out=None, ws=N
     if ws is None:
         ws = torch.empty(exl3_moe_ws(R, H, I, table.E, topk), dtype=torch.uint8, device=x.device)
         ws_clean = False
-    flags = (1 if ws_clean else 0) | (2 if multi_kernel else 0) | (4 if getattr(table, "mixed", False) else 0)
+    flags = (1 if ws_clean else 0) | (2 if multi_kernel else 0) | (4 if getattr(table, "mixed", False) else 0) | (8 if getattr(table, "varw", False) else 0)
     _ck(_lib().spark_exl3_moe(_p(x), _XT[x.dtype], x.stride(0), R, _p(_dev(idx)), int(idx.dtype == torch.int64), _p(_dev(w)), int(w.dtype == torch.float16),
                               _p(table.tab), _p(add), _p(out), _p(ws), H, I, table.E, topk, codebook, act, flags, _st()), "spark_exl3_moe")
     return out
@@ -466,6 +471,15 @@ def qwen_moe_experts(x, idx, w, table, add=None, S=4):
     ws = torch.empty(_lib().qwen_moe_ws_bytes(R, S), dtype=torch.uint8, device=x.device)
     out = torch.empty(R, 2560, dtype=torch.float32, device=x.device)
     _ck(_lib().qwen_moe_experts(_p(x), x.stride(0), R, _p(_dev(idx)), _p(_dev(w)), _p(table.tab), _p(add), _p(out), _p(ws), S, _st()), "qwen_moe_experts")
+    return out
+
+
+def glm_moe3_experts(x, idx, w, table, add=None, S=2, kmask=1 << 4):
+    """reference moe_own.rs:44-46 (TP3): as glm_moe_experts with every expert 768 or 640 wide (table rows 9 and 10)."""
+    R = x.shape[0]
+    ws = torch.empty(_lib().glm_moe3_ws_bytes(R, S), dtype=torch.uint8, device=x.device)
+    out = torch.empty(R, 4096, dtype=torch.float32, device=x.device)
+    _ck(_lib().glm_moe3_experts(_p(x), x.stride(0), R, _p(_dev(idx)), _p(_dev(w)), _p(table.tab), _p(add), _p(out), _p(ws), S, kmask, _st()), "glm_moe3_experts")
     return out
 
 

@@ -170,6 +170,31 @@ def test_glm_mixed_widths_through_kmask(ops, oracle):
         ops.glm_moe_experts(dev_f16(x16.view(np.uint16)), dev(idx8), dev_f16(w8.view(np.uint16)), t, kmask=1 << 7)
 
 
+def test_glm_three_way_split_widths(ops, oracle):
+    # glm_moe3_experts: every expert 768 or 640 wide (row 10 of the table), intermediates strided by the widest
+    g = synth.rng(480)
+    R, E, H = 2, 288, 4096
+    idx8 = np.stack([g.permutation(E)[:8] for _ in range(R)]).astype(np.int64)
+    used = sorted(set(idx8.ravel().tolist()))
+    widths = {e: 768 if k % 3 == 0 else 640 for k, e in enumerate(used)}
+    experts = {e: synth.exl3_expert(g, H, widths[e], 4) for e in used}
+    w8 = (g.uniform(0, 1, (R, 8)) + 0.1).astype(np.float16)
+    x16 = g.standard_normal((R, H)).astype(np.float16)
+    t = ops.ExpertTable(_to_dev(experts), E, widths=widths)
+    out = host(ops.glm_moe3_experts(dev_f16(x16.view(np.uint16)), dev(idx8), dev_f16(w8.view(np.uint16)), t))
+    ref = np.zeros((R, H), np.float32)
+    wid = np.vectorize(widths.get)(idx8)
+    for wd in (640, 768):
+        sel = {e: experts[e] for e in used if widths[e] == wd}
+        w_b = np.where(wid == wd, w8.astype(np.float32), 0.0).astype(np.float32)
+        idx_b = np.where(wid == wd, idx8, next(iter(sel))).astype(np.int32)
+        ref += oracle.exl3_moe(x16.astype(np.float32), idx_b, w_b, sel, E, H, wd, 4, 1, 1)
+    assert rel_l2(out, ref) <= TOL, rel_l2(out, ref)
+    # the run-time-sized entry point with the same table (flags bit 3)
+    out2 = host(ops.exl3_moe(dev_f16(x16.view(np.uint16)), dev(idx8), dev_f16(w8.view(np.uint16)), t, H, 768, codebook=1, act=1))
+    assert np.array_equal(out, out2)
+
+
 def test_exl3_moe_rejects_bad_shapes(ops):
     x = torch.zeros(1, 200, device=DEV)
     with pytest.raises(ops.KernelError):
