@@ -135,6 +135,49 @@ __device__ __forceinline__ void fwht128(float& v0, float& v1, int lane)
     v1 *= 0.08838834764831845f;
 }
 
+// ---- the items of a routed call, worked out by ONE wave.  Items are the call's distinct experts in order of first appearance;
+// an item's pairs are the (row, slot) pairs routed to its expert, ascending.  Lane l holds pairs l, l + 64, ... (NJ per lane).
+// owner: LDS scratch with one int per expert id.  No barrier inside: LDS operations of one wave execute in order.
+template <int NJ> struct WaveItems { int e[NJ]; bool first[NJ]; int rank[NJ]; };
+__device__ __forceinline__ int lanes_below(uint64_t m) { return (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u)); }
+template <int NJ, class F> __device__ __forceinline__ void wave_items_init(WaveItems<NJ>& w, int P, int lane, int* owner, F expert_of)
+{
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) { const int p = lane + 64 * j; w.e[j] = p < P ? expert_of(p) : -1; }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) if (w.e[j] >= 0) owner[w.e[j]] = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) if (w.e[j] >= 0) atomicMin(&owner[w.e[j]], lane + 64 * j);
+    int base = 0;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        w.first[j] = w.e[j] >= 0 && owner[w.e[j]] == lane + 64 * j;      // the first pair of its expert
+        const uint64_t m = __builtin_amdgcn_ballot_w64(w.first[j]);
+        w.rank[j] = base + lanes_below(m);
+        base += __builtin_popcountll(m);
+    }
+}
+// item g: its expert (or -1 when the call has fewer items), its pairs in rows[0 .. n)
+template <int NJ> __device__ __forceinline__ int wave_items_pick(const WaveItems<NJ>& w, int g, int lane, int* rows, int& n)
+{
+    int eg = -1;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const uint64_t m = __builtin_amdgcn_ballot_w64(w.first[j] && w.rank[j] == g);
+        if (m) eg = __shfl(w.e[j], __builtin_ctzll(m), 64);
+    }
+    n = 0;
+    if (eg < 0) return -1;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const bool hit = w.e[j] == eg;
+        const uint64_t m = __builtin_amdgcn_ballot_w64(hit);
+        if (hit) rows[n + lanes_below(m)] = lane + 64 * j;
+        n += __builtin_popcountll(m);
+    }
+    return eg;
+}
+
 // 16-byte streaming load (weights are read once: keep them out of the way of reused data)
 __device__ __forceinline__ uint4 ld_stream16(const void* p)
 {

@@ -49,6 +49,7 @@ constexpr int TWB = 4;                // k-tiles per wave of a stage-2 block (al
 constexpr int TWMAX = 8;              // most k-tiles per wave of a stage-1 block (4 or 8, chosen per shape)
 constexpr int PF_MAX = 256, RF_MAX = 16;
 constexpr int SPIN_MAX = 200000;
+constexpr int EMAX_F = 1024;           // most experts of a layer on this path
 constexpr int SMAX = 8;               // K slices per product (K <= 4096)
 constexpr int NXCD = 8;
 constexpr int HEAD = 256;             // bytes at the start of the workspace: [0] error flag (sticky)
@@ -128,9 +129,9 @@ __device__ __forceinline__ void cvt_x2(int xtype, uint32_t r0, uint32_t r1, floa
 }
 
 struct Group { int e, n; };
-// item g of the call: expert and its pair rows (ascending), or n = 0 when the call has fewer items.  All threads call.
-// Leaves every pair's expert in sidx[] when R > 1.
-__device__ __forceinline__ Group find_item(const FArgs& a, int g, int* sidx, unsigned char* isf, int* rows, int* misc)
+// item g of the call: expert and its pair rows (ascending) in rows[], or n = 0 when the call has fewer items.  All threads
+// call; wave 0 works the item out (one barrier).  Leaves every pair's expert in sidx[] when R > 1.
+__device__ __forceinline__ Group find_item(const FArgs& a, int g, int* sidx, int* owner, int* rows, int* misc)
 {
     const int P = a.P, tid = threadIdx.x;
     if (a.R == 1) {                                       // every pair is its own item
@@ -139,34 +140,17 @@ __device__ __forceinline__ Group find_item(const FArgs& a, int g, int* sidx, uns
         __syncthreads();
         return Group{exl3_ld_idx(a.idx, a.c.itype, g), 1};
     }
-    if (tid == 0) { misc[0] = -1; misc[1] = 0; }
-    for (int p = tid; p < P; p += blockDim.x) sidx[p] = exl3_ld_idx(a.idx, a.c.itype, p);
-    __syncthreads();
-    for (int p = tid; p < P; p += blockDim.x) {           // first occurrence of its expert?
-        const int e = sidx[p];
-        bool first = true;
-        for (int q = 0; q < p; ++q) first &= sidx[q] != e;
-        isf[p] = first;
+    if (tid < 64) {
+        WaveItems<PF_MAX / 64> wi;
+        wave_items_init(wi, P, tid, owner, [&](int p) { return exl3_ld_idx(a.idx, a.c.itype, p); });
+#pragma unroll
+        for (int j = 0; j < PF_MAX / 64; ++j) if (tid + 64 * j < P) sidx[tid + 64 * j] = wi.e[j];
+        int n = 0;
+        const int e = wave_items_pick(wi, g, tid, rows, n);
+        if (tid == 0) { misc[0] = e; misc[1] = n; }
     }
     __syncthreads();
-    for (int p = tid; p < P; p += blockDim.x)
-        if (isf[p]) {
-            int before = 0;
-            for (int q = 0; q < p; ++q) before += isf[q];
-            if (before == g) misc[0] = sidx[p];
-        }
-    __syncthreads();
-    const int e = misc[0];
-    if (e < 0) return Group{0, 0};
-    for (int p = tid; p < P; p += blockDim.x)
-        if (sidx[p] == e) {
-            int slot = 0;
-            for (int q = 0; q < p; ++q) slot += sidx[q] == e;
-            rows[slot] = p;
-            atomicAdd(&misc[1], 1);
-        }
-    __syncthreads();
-    return Group{e, misc[1]};
+    return misc[0] < 0 ? Group{0, 0} : Group{misc[0], misc[1]};
 }
 
 template <int CBK, int MR, int TWA, bool LOCAL>
@@ -176,7 +160,7 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
     __shared__ float red[FW][MR][128];
     __shared__ int sidx[PF_MAX], rows[RF_MAX], comb[RF_MAX], misc[4];
     __shared__ float wsh[RF_MAX][16];                     // route weights of this item's token rows (stage 2)
-    __shared__ unsigned char isf[PF_MAX];
+    __shared__ int owner[EMAX_F];                         // one int per expert id: scratch of the item lookup
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bid = blockIdx.x;
     const bool isA = bid < a.nA;
@@ -206,7 +190,7 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
     }
     if (tid == 0) misc[2] = 1;
     Group grp{0, 0};
-    if (g >= 0) grp = find_item(a, g, sidx, isf, rows, misc);
+    if (g >= 0) grp = find_item(a, g, sidx, owner, rows, misc);
     TRACE(1);
     if (grp.n > 0) {
         const int Kt = K / 16, Nt = N / 16;
@@ -535,7 +519,7 @@ int g_xcd_local = -1;                 // -1 unknown, 0 placement check failed, 1
 
 bool exl3_fused_ok(const Exl3Cfg& c, int R)
 {
-    return R >= 1 && R <= RF_MAX && c.topk <= 16 && R * c.topk <= PF_MAX && c.H <= SMAX * FW * TWMAX * 16 && c.I <= SMAX * FW * TWB * 16;
+    return R >= 1 && R <= RF_MAX && c.E <= EMAX_F && c.topk <= 16 && R * c.topk <= PF_MAX && c.H <= SMAX * FW * TWMAX * 16 && c.I <= SMAX * FW * TWB * 16;
 }
 size_t exl3_fused_ws_bytes(const Exl3Cfg& c, int R) { return fplan(c, R).total; }
 

@@ -74,53 +74,13 @@ __device__ __forceinline__ int pair_expert(const MArgs& a, int p)
     const int r = p / a.TT, k = p % a.TT;
     return k < a.topk ? (int)a.idx[(int64_t)r * a.topk + k] : a.E + (k - a.topk);
 }
-struct Group { int e, n; };
-// item g of the call (distinct experts in order of first appearance): expert and its pairs (ascending) in rows[]
-__device__ __forceinline__ Group find_item(const MArgs& a, int g, int* sidx, unsigned char* isf, int* rows, int* misc)
-{
-    const int P = a.P, tid = threadIdx.x;
-    if (a.R == 1) {
-        if (g >= P) return Group{0, 0};
-        if (tid == 0) rows[0] = g;
-        __syncthreads();
-        return Group{pair_expert(a, g), 1};
-    }
-    if (tid == 0) { misc[0] = -1; misc[1] = 0; }
-    for (int p = tid; p < P; p += NT) sidx[p] = pair_expert(a, p);
-    __syncthreads();
-    for (int p = tid; p < P; p += NT) {
-        const int e = sidx[p];
-        bool first = true;
-        for (int q = 0; q < p; ++q) first &= sidx[q] != e;
-        isf[p] = first;
-    }
-    __syncthreads();
-    for (int p = tid; p < P; p += NT)
-        if (isf[p]) {
-            int before = 0;
-            for (int q = 0; q < p; ++q) before += isf[q];
-            if (before == g) misc[0] = sidx[p];
-        }
-    __syncthreads();
-    const int e = misc[0];
-    if (e < 0) return Group{0, 0};
-    for (int p = tid; p < P; p += NT)
-        if (sidx[p] == e) {
-            int slot = 0;
-            for (int q = 0; q < p; ++q) slot += sidx[q] == e;
-            rows[slot] = p;
-            atomicAdd(&misc[1], 1);
-        }
-    __syncthreads();
-    return Group{e, misc[1]};
-}
+struct Group { int e, n; };      // an item: expert and number of pairs (rows), the pairs ascending in a rows[] array
 
 template <int LAYOUT, bool QUANT, bool LOCAL>
 __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ int sidx[PMAXF], rowsU[RMAX], rowsD[RMAX], comb[RMAX], misc[4];
-    __shared__ unsigned char isf[PMAXF];
+    __shared__ int sidx[PMAXF], rowsU[RMAX], rowsD[RMAX], comb[RMAX], misc[4], gsel[4];
     __shared__ float amx[NW][16];
     __shared__ __align__(16) uint32_t hbw[16][8];          // the block's 32 code bytes per item row
     __shared__ uint32_t he[16];
@@ -134,11 +94,29 @@ __global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
     TRACE(0);
     __builtin_amdgcn_s_setprio(2);
     const bool hasU = grpi < a.Gmax && bi < a.NJ;
-    // both items of this block up front: the stage-2 loads must not wait for an index lookup later
+    // both items of this block up front (the stage-2 loads must not wait for an index lookup later), worked out by one wave
     Group gu{0, 0}, gd{0, 0};
-    if (hasU) gu = find_item(a, grpi, sidx, isf, rowsU, misc);
-    __syncthreads();
-    if (grpi >= 1 && bi < a.NBD) gd = find_item(a, grpi - 1, sidx, isf, rowsD, misc);
+    const bool wantU = hasU, wantD = grpi >= 1 && bi < a.NBD;
+    if (a.R == 1) {                                        // every pair is its own item
+        if (wantU && grpi < a.P) gu = Group{pair_expert(a, grpi), 1};
+        if (wantD && grpi - 1 < a.P) gd = Group{pair_expert(a, grpi - 1), 1};
+        if (tid == 0) { rowsU[0] = grpi; rowsD[0] = grpi - 1; }
+        __syncthreads();
+    } else {
+        if (wave == 0) {
+            WaveItems<PMAXF / 64> wi;
+            wave_items_init(wi, a.P, lane, (int*)smem, [&](int p) { return pair_expert(a, p); });
+#pragma unroll
+            for (int j = 0; j < PMAXF / 64; ++j) if (lane + 64 * j < a.P) sidx[lane + 64 * j] = wi.e[j];
+            int nu = 0, nd = 0;
+            const int eu = wantU ? wave_items_pick(wi, grpi, lane, rowsU, nu) : -1;
+            const int ed = wantD ? wave_items_pick(wi, grpi - 1, lane, rowsD, nd) : -1;
+            if (lane == 0) { gsel[0] = eu; gsel[1] = nu; gsel[2] = ed; gsel[3] = nd; }
+        }
+        __syncthreads();
+        gu = Group{gsel[0], gsel[0] >= 0 ? gsel[1] : 0};
+        gd = Group{gsel[2], gsel[2] >= 0 ? gsel[3] : 0};
+    }
     TRACE(1);
     if (gu.n > 0) {
         // ================================================================ stage 1
