@@ -48,6 +48,8 @@ class Exl3Layer:
     """Config 2: EXL3 4-bit, H 2048, I 512, 512 experts top-10 (mul1 codebook)."""
     H, I, E, TOPK, LAYERS = 2048, 512, 512, 10, 48
     BYTES_PER_EXPERT = 3 * 524288 + 3 * (2048 + 512) * 2        # trellis + suh/svh (fp16)
+    DTYPE = "f16 (4-bit trellis codes decoded to fp16 codebook values, fp32 accumulate)"
+    SET = "805 MB expert set"
 
     def __init__(self, torch, ops, R, inst, seed=0):
         self.torch, self.ops, self.R, self.inst = torch, ops, R, inst
@@ -118,6 +120,8 @@ class Mxfp4Layer:
     """Config 3: MXFP4 experts, H 4096, I 2048, 384 experts top-6 + 1 shared (sqrt-softplus router)."""
     H, I, E, TOPK, NS, LAYERS = 4096, 2048, 384, 6, 1, 61
     BYTES_PER_EXPERT = 3 * (4194304 + 262144)
+    DTYPE = "fp4 x fp8 (E2M1 weights x E4M3 activations, E8M0 block scales, block-scaled MFMA, fp32 accumulate)"
+    SET = "5.1 GB expert set"
 
     def __init__(self, torch, ops, R, inst, seed=1):
         self.torch, self.ops, self.R, self.inst = torch, ops, R, inst
@@ -195,6 +199,8 @@ class Mxfp4Prefill(Mxfp4Layer):
 class Fp8Dense:
     """Config 4: FP8 E4M3 dense projection with 128x128 FP32 block scales."""
     LAYERS = 1
+    DTYPE = "fp8 x bf16 (E4M3 weights, fp32 block scales, fp32 accumulate)"
+    SET = "rotating over more than 512 MB of weight copies"
 
     def __init__(self, torch, ops, R, inst, N, K, seed=2):
         self.torch, self.ops, self.R, self.inst, self.N, self.K = torch, ops, R, inst, N, K
@@ -298,6 +304,7 @@ def main():
         wl = Mxfp4Prefill(torch, ops, 2048, INST)
     else:
         wl = Fp8Dense(torch, ops, a.batch, INST, *((7168, 4096) if a.config == "c4a" else (4096, 7168)))
+    dtype, wset = wl.DTYPE, wl.SET
     ms = time_steps(torch, wl, a.steps, a.warmup, INST)
     head = line_for(wl, ms)
     # the dominant kernel alone, same graphs and events: its average launch duration prices the roofline
@@ -334,8 +341,8 @@ def main():
     out = {
         "metric": "us per MoE layer (+ achieved HBM GB/s, % of peak) at batch 1/4", "value": head["us_per_layer"], "unit": "us per MoE layer",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "u4 trellis codes -> fp16 codebook, fp32 accumulate", "data": "synthetic",
-        "config": {"workload": head["workload"], "timing": f"HIP graph of {INST} layer instances with fresh routes, weights cold (805 MB expert set)",
+        "dtype": dtype, "data": "synthetic",
+        "config": {"workload": head["workload"], "timing": f"HIP graph of {INST} layer instances with fresh routes, weights cold ({wset})",
                    "tok_per_s_equiv": head["tok_per_s_equiv"], "layers_assumed": head["layers_assumed"]},
         "roofline": {"bound": "hbm", "achieved": round(k_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(k_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get((a.config, a.batch)),
                      "kernel": k_name, "kernel_us_per_launch": round(k_us, 3), "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
