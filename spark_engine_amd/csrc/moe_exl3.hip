@@ -284,9 +284,10 @@ inline Plan plan(const Cfg& c, int R)
 {
     Plan p;
     p.P = R * c.topk;
-    p.Gmax = p.P < c.E ? p.P : c.E;
-    p.S1 = slices(c.H / 16, (c.I / 128) * 2 * p.Gmax);
-    p.S2 = slices(c.I / 16, (c.H / 128) * p.Gmax);
+    p.Gmax = (p.P < c.E ? p.P : c.E) + p.P / 16;        // items: an expert's rows go 16 to an item (the last one short)
+    // the K slices depend on the shape only (sized for 16 items): a row's summation order, and so its bits, are the same in every call
+    p.S1 = slices(c.H / 16, (c.I / 128) * 2 * 16);
+    p.S2 = slices(c.I / 16, (c.H / 128) * 16);
     size_t o = 0;
     auto take = [&](size_t n) { const size_t q = o; o += align256(n); return q; };
     p.G = take(16);
@@ -357,6 +358,26 @@ int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, co
     return launch_status();
 }
 
+// Calls with more rows than one pass takes (64 rows, 1024 pairs) run pass after pass over row ranges: a row's result does not
+// depend on the other rows of a call, so the values are those of one big call.  The passes share the workspace.
+inline int rows_per_pass(const Cfg& c) { const int byp = PMAX / c.topk; return byp < 64 ? byp : 64; }
+int experts_rows(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
+                 int flags, hipStream_t st)
+{
+    if (R < 1 || c.topk < 1 || c.topk > 64) return -1;
+    const int RC = rows_per_pass(c);
+    if (R <= RC) return experts(c, x, ldx, R, idx, w, tab, add, out, ws, flags, st);
+    const size_t xsz = c.xtype == X_F32 ? 4 : 2, isz = c.itype ? 8 : 4, wsz = c.wtype ? 2 : 4;
+    for (int r0 = 0; r0 < R; r0 += RC) {
+        const int n = R - r0 < RC ? R - r0 : RC;
+        const int rc = experts(c, (const char*)x + (size_t)r0 * ldx * xsz, ldx, n, (const char*)idx + (size_t)r0 * c.topk * isz,
+                               (const char*)w + (size_t)r0 * c.topk * wsz, tab, add ? (const float*)add + (size_t)r0 * c.H : nullptr,
+                               (float*)out + (size_t)r0 * c.H, ws, flags & ~1, st);      // a pass of another size leaves other words behind: no "prepared" promise
+        if (rc) return rc;
+    }
+    return 0;
+}
+
 const Cfg QWEN{512, 10, 2560, 640, CB_MUL1, 0, X_F32, 0, 0};
 const Cfg GLM{288, 8, 4096, 1024, CB_MCG, 1, X_F16, 1, 1};
 const Cfg GLM3{288, 8, 4096, 768, CB_MCG, 1, X_F16, 1, 1};        // TP3: experts 640 or 768 wide, I = the widest (strides)
@@ -367,15 +388,21 @@ const Cfg GLM3{288, 8, 4096, 768, CB_MCG, 1, X_F16, 1, 1};        // TP3: expert
 
 // Runtime-sized entry (no reference counterpart symbol): x [R, H] of xtype (0 f32, 1 f16, 2 bf16), row stride ldx;
 // idx [R, topk] int32 (itype 0) or int64 (1); w [R, topk] f32 (wtype 0) or f16 (1); tab u64 [9][E]; codebook 2 = mul1,
-// 1 = mcg; act 0 = silu(g) u, 1 = clamped; add / out f32 [R, H].  4-bit trellis, R <= 64 rows.
+// 1 = mcg; act 0 = silu(g) u, 1 = clamped; add / out f32 [R, H].  Any R: more than 64 rows (1024 pairs) run as several passes.
 // flags bit 0: the workspace was zeroed by spark_exl3_moe_ws_init and only used by this entry since (saves a launch);
 // bit 1: use the multi-kernel path even where the single-launch path applies.
 SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk)
 {
     const Cfg c{E, topk, H, I, CB_MUL1, 0, 0, 0, 0};
-    if (!cfg_ok(c, R)) return 0;
-    const size_t a = plan(c, R).total, b = exl3_fused_ok(c, R) ? exl3_fused_ws_bytes(c, R) : 0;
-    return a + b;
+    if (R < 1 || topk < 1 || topk > 64) return 0;
+    const int RC = rows_per_pass(c);
+    auto one = [&](int n) -> size_t {
+        if (n < 1 || !cfg_ok(c, n)) return 0;
+        return plan(c, n).total + (exl3_fused_ok(c, n) ? exl3_fused_ws_bytes(c, n) : 0);
+    };
+    if (R <= RC) return one(R);
+    const size_t a = one(RC), b = one(R % RC);       // the full passes and the last, shorter one
+    return a == 0 ? 0 : (a > b ? a : b);
 }
 // prepares the workspace once after allocation; calls made with flags bit 0 set then skip their own preparing launch
 SPARK_API int spark_exl3_moe_ws_init(void* ws, size_t bytes, hipStream_t st)
@@ -387,7 +414,7 @@ SPARK_API int spark_exl3_moe(const void* x, int xtype, int64_t ldx, int R, const
                              const void* add, void* out, void* ws, int H, int I, int E, int topk, int codebook, int act, int flags, hipStream_t st)
 {
     const Cfg c{E, topk, H, I, codebook, act, xtype, wtype, itype};
-    return experts(c, x, ldx, R, idx, w, tab, add, out, ws, flags, st);
+    return experts_rows(c, x, ldx, R, idx, w, tab, add, out, ws, flags, st);
 }
 // reference qwen_moe.cu:112-116: x f32 [R, 2560], idx i32 / w f32 [R, 10], tab u64 [9][512], out f32 [R, 2560]; S is the
 // reference's K-slice hint (the slice count is chosen from the shape here)
@@ -396,7 +423,7 @@ SPARK_API int qwen_moe_experts(const void* x, int64_t ldx, int R, const void* id
                                hipStream_t st)
 {
     (void)S;
-    return experts(QWEN, x, ldx, R, idx, w, tab, add, out, ws, 0, st);
+    return experts_rows(QWEN, x, ldx, R, idx, w, tab, add, out, ws, 0, st);
 }
 // reference glm_moe.cu:6-24: x f16 [R, 4096], idx i64 / w f16 [R, 8], tab u64 [10|11][288] (rows 0-8 as above), mcg codebook,
 // clamped SwiGLU.  suh0 (shared gate/up input scales) is a prefill shortcut and is not needed.  kmask = bit K set for every
@@ -407,7 +434,7 @@ SPARK_API int glm_moe_experts(const void* x, int64_t ldx, int R, const void* idx
 {
     (void)S; (void)suh0;
     if (kmask <= 0 || (kmask & ~0x78)) return -4;              // widths 3..6 only
-    return experts(GLM, x, ldx, R, idx, w, tab, add, out, ws, kmask == (1 << 4) ? 0 : 4, st);
+    return experts_rows(GLM, x, ldx, R, idx, w, tab, add, out, ws, kmask == (1 << 4) ? 0 : 4, st);
 }
 // reference glm_moe.cu:17-24 (moex::GlmMoe3, moe_exl3.cuh:63-67): GLM under a three-way split, every expert 768 or 640 wide (6 or
 // 5 of its 128-wide Hadamard blocks); tab u64 [11][288]: rows 0-8 as above, row 9 the trellis width in bits, row 10 the
@@ -418,5 +445,5 @@ SPARK_API int glm_moe3_experts(const void* x, int64_t ldx, int R, const void* id
 {
     (void)S;
     if (kmask <= 0 || (kmask & ~0x78)) return -4;
-    return experts(GLM3, x, ldx, R, idx, w, tab, add, out, ws, 8 | (kmask == (1 << 4) ? 0 : 4), st);
+    return experts_rows(GLM3, x, ldx, R, idx, w, tab, add, out, ws, 8 | (kmask == (1 << 4) ? 0 : 4), st);
 }

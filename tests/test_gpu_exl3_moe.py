@@ -195,6 +195,22 @@ def test_glm_three_way_split_widths(ops, oracle):
     assert np.array_equal(out, out2)
 
 
+def test_exl3_moe_prefill_sized_call(ops, oracle):
+    # more rows than one pass takes: the call runs pass after pass over row ranges, the last one short
+    g = synth.rng(490)
+    R, H, I, E, topk = 150, 256, 128, 6, 2
+    experts = _layer(g, range(E), H, I)
+    idx = np.stack([g.permutation(E)[:topk] for _ in range(R)]).astype(np.int32)
+    w = g.uniform(0.1, 1.0, (R, topk)).astype(np.float32)
+    x = g.standard_normal((R, H)).astype(np.float32)
+    add = g.standard_normal((R, H)).astype(np.float32)
+    table = ops.ExpertTable(_to_dev(experts), E)
+    out = host(ops.exl3_moe(dev(x), dev(idx), dev(w), table, H, I, add=dev(add)))
+    assert rel_l2(out, oracle.exl3_moe(x, idx, w, experts, E, H, I, 4, 2, 0, add=add)) <= TOL
+    one = host(ops.exl3_moe(dev(x[140:141]), dev(idx[140:141]), dev(w[140:141]), table, H, I, add=dev(add[140:141]), multi_kernel=True))
+    assert np.array_equal(one[0], out[140])                           # a row of the short last pass (several-kernel path), alone
+
+
 def test_exl3_moe_rejects_bad_shapes(ops):
     x = torch.zeros(1, 200, device=DEV)
     with pytest.raises(ops.KernelError):
