@@ -80,12 +80,55 @@ __global__ __launch_bounds__(256) void had_kernel(const void* __restrict__ x, in
     const uint16_t* suh = (const uint16_t*)tab[(int64_t)(suh_slot0 + t) * E + pexp[row]];
     const int64_t src = prow[row];
     const int k = kb * 128 + lane * 2;
-    float v0 = ld_x(x, xtype, src * ldx + k) * f16_bits_to_f32(suh[k]);
-    float v1 = ld_x(x, xtype, src * ldx + k + 1) * f16_bits_to_f32(suh[k + 1]);
+    // the lane's two elements in one access each (rows start on even elements: ldx is even for every caller's layout)
+    float v0, v1;
+    if (xtype == X_F32) { const float2 xv = *(const float2*)((const float*)x + src * ldx + k); v0 = xv.x; v1 = xv.y; }
+    else {
+        const uint32_t xv = *(const uint32_t*)((const uint16_t*)x + src * ldx + k);
+        if (xtype == X_F16) { v0 = f16_bits_to_f32((uint16_t)xv); v1 = f16_bits_to_f32((uint16_t)(xv >> 16)); }
+        else { v0 = __uint_as_float(xv << 16); v1 = __uint_as_float(xv & 0xffff0000u); }
+    }
+    const uint32_t sv = *(const uint32_t*)(suh + k);
+    v0 *= f16_bits_to_f32((uint16_t)sv); v1 *= f16_bits_to_f32((uint16_t)(sv >> 16));
     fwht128(v0, v1, lane);
-    uint16_t* d = xh + ((int64_t)t * P + row) * K + k;
-    d[0] = f32_to_f16_bits(v0);
-    d[1] = f32_to_f16_bits(v1);
+    *(uint32_t*)(xh + ((int64_t)t * P + row) * K + k) = (uint32_t)f32_to_f16_bits(v0) | ((uint32_t)f32_to_f16_bits(v1) << 16);
+}
+
+// the same transform for prefill-sized calls: wave per (t, row), all 128-blocks of the row with their loads in flight together
+// (one wave per 128-block leaves every wave alone with a chain of dependent lookups)
+__global__ __launch_bounds__(256) void had_rows_kernel(const void* __restrict__ x, int xtype, int64_t ldx, const uint64_t* __restrict__ tab, int E,
+                                                       int suh_slot0, int T, int P, const int* __restrict__ prow, const int* __restrict__ pexp, int K,
+                                                       uint16_t* __restrict__ xh)
+{
+    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63;
+    const int row = (int)(wave % P), t = (int)(wave / P);
+    if (t >= T) return;
+    const uint16_t* suh = (const uint16_t*)tab[(int64_t)(suh_slot0 + t) * E + pexp[row]];
+    const int64_t src = prow[row];
+    uint16_t* dst = xh + ((int64_t)t * P + row) * K;
+    for (int kb0 = 0; kb0 < K / 128; kb0 += 4) {
+        float v0[4], v1[4];
+        uint32_t sv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int k = min(kb0 + u, K / 128 - 1) * 128 + lane * 2;
+            if (xtype == X_F32) { const float2 xv = *(const float2*)((const float*)x + src * ldx + k); v0[u] = xv.x; v1[u] = xv.y; }
+            else {
+                const uint32_t xv = *(const uint32_t*)((const uint16_t*)x + src * ldx + k);
+                if (xtype == X_F16) { v0[u] = f16_bits_to_f32((uint16_t)xv); v1[u] = f16_bits_to_f32((uint16_t)(xv >> 16)); }
+                else { v0[u] = __uint_as_float(xv << 16); v1[u] = __uint_as_float(xv & 0xffff0000u); }
+            }
+            sv[u] = *(const uint32_t*)(suh + k);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (kb0 + u >= K / 128) break;
+            float a = v0[u] * f16_bits_to_f32((uint16_t)sv[u]), b = v1[u] * f16_bits_to_f32((uint16_t)(sv[u] >> 16));
+            fwht128(a, b, lane);
+            *(uint32_t*)(dst + (kb0 + u) * 128 + lane * 2) = (uint32_t)f32_to_f16_bits(a) | ((uint32_t)f32_to_f16_bits(b) << 16);
+        }
+    }
 }
 
 // ---------------------------------------------------------------- the weight stream: partial GEMV of one item
@@ -276,6 +319,163 @@ __global__ __launch_bounds__(256) void finish_combine_kernel(const float* __rest
     out[(int64_t)r * H + n + 1] = b1 + a1;
 }
 
+// ================================================================ prefill: grouped GEMM over 64-row items
+// With many rows per expert the GEMV path decodes every weight once per 16 rows; here a block owns 64 item rows x 128 output
+// columns for the whole K range and decodes each weight once: per chunk of 128 K the four waves decode their k-tiles into LDS as
+// fp16 ([column][k]), the item's transformed activation rows are staged next to them, and every wave multiplies its 32 columns
+// with v_mfma_f32_16x16x16_f16 (weights = A, activations = B: a lane ends up with four neighbouring columns of one row, a 16-byte
+// store; binary32 accumulate).  The next chunk's loads are in flight during
+// the multiplies.  reference moe_exl3.cuh:520-1370 (gux_kernel, gemm_grouped_kernel): decode once, tensor-core multiply.
+constexpr int PG_ROWS = 64;            // rows of a prefill item
+constexpr int PG_KT = 4;              // k-tiles per chunk of the grouped GEMM
+constexpr int EBIG = 1024;             // experts the prefill grouping holds
+
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+// pairs -> items of at most GR rows per expert (rows of an expert in no particular order: every row is computed on its own)
+__global__ __launch_bounds__(1024) void prep_big_kernel(const void* __restrict__ idx, int itype, int R, int topk, int E, int GR, int* __restrict__ G,
+                                                       int* __restrict__ gexp, int* __restrict__ goff, int* __restrict__ gcnt, int* __restrict__ pairmap,
+                                                       int* __restrict__ prow, int* __restrict__ pexp)
+{
+    __shared__ int cnt[EBIG], fill[EBIG], eoff[EBIG], ioff[EBIG];
+    __shared__ int wsum[2][16];
+    const int tid = threadIdx.x, P = R * topk;
+    if (tid < E) { cnt[tid] = 0; fill[tid] = 0; }
+    __syncthreads();
+    for (int p0 = tid; p0 < P; p0 += 8 * 1024) {
+        int ev[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) ev[u] = ld_idx(idx, itype, min(p0 + u * 1024, P - 1));
+#pragma unroll
+        for (int u = 0; u < 8; ++u) if (p0 + u * 1024 < P) atomicAdd(&cnt[ev[u]], 1);
+    }
+    __syncthreads();
+    const int c = tid < E ? cnt[tid] : 0, nit = (c + GR - 1) / GR;
+    int rs = c, is = nit;
+    const int lane = tid & 63, wv = tid >> 6;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int a = __shfl_up(rs, o, 64), b = __shfl_up(is, o, 64);
+        if (lane >= o) { rs += a; is += b; }
+    }
+    if (lane == 63) { wsum[0][wv] = rs; wsum[1][wv] = is; }
+    __syncthreads();
+    int rb = 0, ib = 0;
+    for (int w = 0; w < wv; ++w) { rb += wsum[0][w]; ib += wsum[1][w]; }
+    if (tid == 1023) *G = ib + is;
+    if (tid < E) {
+        eoff[tid] = rb + rs - c; ioff[tid] = ib + is - nit;
+        for (int j = 0; j * GR < c; ++j) { const int it = ib + is - nit + j; gexp[it] = tid; goff[it] = rb + rs - c + j * GR; gcnt[it] = min(GR, c - j * GR); }
+    }
+    __syncthreads();
+    for (int p0 = tid; p0 < P; p0 += 8 * 1024) {
+        int ev[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) ev[u] = ld_idx(idx, itype, min(p0 + u * 1024, P - 1));
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int p = p0 + u * 1024;
+            if (p < P) {
+                const int pos = eoff[ev[u]] + atomicAdd(&fill[ev[u]], 1);
+                pairmap[p] = pos; prow[pos] = p / topk; pexp[pos] = ev[u];
+            }
+        }
+    }
+}
+
+// grid (N / 128, 1, T * Gmax), 4 waves.  xh [T][P][K] fp16 (rows = compact pair rows), part [T][P][N] binary32.
+// KT = k-tiles per chunk (4 or 8): the smaller chunk halves the LDS of a block, so more blocks share a CU.
+template <int CBK, int KT>
+__global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ xh, const uint64_t* __restrict__ tab, int E, int tr_slot0,
+                                                   const int* __restrict__ G, const int* __restrict__ gexp, const int* __restrict__ goff,
+                                                   const int* __restrict__ gcnt, int Gmax, int T, int P, int K, int N, float* __restrict__ part)
+{
+    constexpr int LD = KT * 16 + 4;                     // halfs per LDS row: the chunk + 4 (8-byte operand reads down a column of rows hit distinct banks)
+    constexpr int TW = KT / 4;                          // k-tiles a wave decodes per chunk
+    constexpr int XV = KT / 2;                          // 16-byte loads per thread of the activation stage (a quarter of the chunk)
+    __shared__ __align__(16) uint16_t wl[128 * LD];     // [column][k of the chunk]
+    __shared__ __align__(16) uint16_t xl[PG_ROWS * LD]; // [row][k of the chunk]
+    const int tg = blockIdx.z, t = tg / Gmax, g = tg % Gmax;
+    if (g >= *G) return;
+    const int rows = gcnt[g];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), c = lane & 15, q = lane >> 4;
+    const int Nt = N / 16, nb = blockIdx.x, nrt = (rows + 15) >> 4, nch = K / (16 * KT);
+    const uint32_t* tr = (const uint32_t*)tab[(int64_t)(tr_slot0 + t) * E + gexp[g]];
+    const int64_t r0 = (int64_t)t * P + goff[g];
+    // staging roles: thread = (row, quarter of the chunk's K); wave = TW of the chunk's k-tiles
+    const int srow = tid >> 2, spart = tid & 3;
+    const uint16_t* xsrc = xh + (r0 + min(srow, rows - 1)) * K + spart * (XV * 8);
+    const uint32_t* wsrc = tr + ((int64_t)(wave * TW) * Nt + nb * 8) * 32 + lane * 4;
+    const int src = tile_prev_lane(lane), tl = lane >> 3, m = lane & 7;
+    uint4 xa[XV], wt[TW];
+#pragma unroll
+    for (int i = 0; i < XV; ++i) xa[i] = *(const uint4*)(xsrc + i * 8);
+#pragma unroll
+    for (int h = 0; h < TW; ++h) wt[h] = ld_stream16(wsrc + (int64_t)h * Nt * 32);
+    v4f acc[4][2];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) acc[rt][nt] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int ch = 0; ch < nch; ++ch) {
+        // ---- this chunk's operands into LDS
+#pragma unroll
+        for (int i = 0; i < XV; ++i) {
+            uint2* d = (uint2*)&xl[srow * LD + spart * (XV * 8) + i * 8];
+            d[0] = make_uint2(xa[i].x, xa[i].y); d[1] = make_uint2(xa[i].z, xa[i].w);
+        }
+#pragma unroll
+        for (int h = 0; h < TW; ++h) {
+            h2 wd[4][4];
+            decode_tile32<CBK>(wt[h], __shfl(wt[h].w, src, 64), wd);
+            // column m of tile tl: k 0..7 = wd[0..3][0], k 8..15 = wd[0..3][1]; column m + 8: wd[..][2], wd[..][3]
+#pragma unroll
+            for (int cc = 0; cc < 2; ++cc) {
+                uint32_t u[8];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { __builtin_memcpy(&u[j], &wd[j][2 * cc], 4); __builtin_memcpy(&u[4 + j], &wd[j][2 * cc + 1], 4); }
+                uint2* d = (uint2*)&wl[(tl * 16 + m + 8 * cc) * LD + (wave * TW + h) * 16];
+                d[0] = make_uint2(u[0], u[1]); d[1] = make_uint2(u[2], u[3]); d[2] = make_uint2(u[4], u[5]); d[3] = make_uint2(u[6], u[7]);
+            }
+        }
+        __syncthreads();
+        // ---- the next chunk's loads, in flight during the multiplies (past the end: the last chunk again, unused)
+        {
+            const int cn = min(ch + 1, nch - 1);
+#pragma unroll
+            for (int i = 0; i < XV; ++i) xa[i] = *(const uint4*)(xsrc + cn * (16 * KT) + i * 8);
+#pragma unroll
+            for (int h = 0; h < TW; ++h) wt[h] = ld_stream16(wsrc + ((int64_t)cn * KT + h) * Nt * 32);
+        }
+        // ---- wave = columns 32 wave .. + 31: D[col][row] += W[col][k] X[k][row], 16 k per instruction
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            v4h b[2];
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) b[nt] = *(const v4h*)&wl[(wave * 32 + nt * 16 + c) * LD + kt * 16 + 4 * q];
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                if (rt < nrt) {
+                    const v4h a = *(const v4h*)&xl[(rt * 16 + c) * LD + kt * 16 + 4 * q];
+#pragma unroll
+                    for (int nt = 0; nt < 2; ++nt) acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x16f16(b[nt], a, acc[rt][nt], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    // D: lane = row c of the row tile, columns 4 q .. 4 q + 3 of the column tile
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+        const int row = rt * 16 + c;
+        if (row < rows) {
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+                *(float4*)(part + (r0 + row) * N + nb * 128 + wave * 32 + nt * 16 + 4 * q) = make_float4(acc[rt][nt][0], acc[rt][nt][1], acc[rt][nt][2], acc[rt][nt][3]);
+        }
+    }
+}
+
 // ---------------------------------------------------------------- host side
 inline int slices(int Kt, int nblocks) { int s = 1; while (s < 8 && nblocks * s < 768 && Kt / (s * 2) >= 8) s *= 2; return s; }
 
@@ -330,7 +530,7 @@ void launch_gemv(const uint16_t* xh, const uint64_t* tab, int E, int slot0, cons
 int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
             int flags, hipStream_t st)
 {
-    if (!cfg_ok(c, R)) return -1;
+    if (!cfg_ok(c, R) || (ldx & 1)) return -1;       // rows start on even elements (two activations per access)
     const bool mixed = (flags & 4) != 0;             // the table has a row 9 with every expert's trellis width (3..6 bits)
     const bool varw = (flags & 8) != 0;              // and a row 10 with every expert's intermediate width (reference moe_exl3.cuh:63-67,132-136)
     if (!(flags & 2) && !mixed && !varw && exl3_fused_ok(c, R)) return exl3_fused_launch(c, x, ldx, R, idx, w, tab, add, out, ws, flags & 1, st);
@@ -358,6 +558,57 @@ int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, co
     return launch_status();
 }
 
+// ---- prefill: R > 64 rows of a uniform 4-bit table
+struct BigPlan { int P, Gmax; size_t G, gexp, goff, gcnt, pairmap, prow, pexp, xh1, part, xh2, total; };
+inline BigPlan big_plan(const Cfg& c, int R)
+{
+    BigPlan p;
+    p.P = R * c.topk;
+    p.Gmax = (p.P < c.E ? p.P : c.E) + p.P / PG_ROWS + 1;
+    size_t o = 0;
+    auto take = [&](size_t n) { const size_t q = o; o += align256(n); return q; };
+    p.G = take(16);
+    p.gexp = take(4 * (size_t)p.Gmax); p.goff = take(4 * (size_t)p.Gmax); p.gcnt = take(4 * (size_t)p.Gmax);
+    p.pairmap = take(4 * (size_t)p.P); p.prow = take(4 * (size_t)p.P); p.pexp = take(4 * (size_t)p.P);
+    p.xh1 = take(2 * (size_t)p.P * c.H * 2);
+    const size_t e1 = (size_t)2 * p.P * c.I, e2 = (size_t)p.P * c.H;
+    p.part = take(4 * (e1 > e2 ? e1 : e2));
+    p.xh2 = take((size_t)p.P * c.I * 2);
+    p.total = o;
+    return p;
+}
+inline bool big_ok(const Cfg& c, int R)
+{
+    return R > 64 && c.E >= 1 && c.E <= EBIG && c.topk >= 1 && c.topk <= 64 && (int64_t)R * c.topk < (1ll << 24) && c.H >= 128 && c.I >= 128 &&
+           c.H % 128 == 0 && c.I % 128 == 0 && (c.cbk == CB_MCG || c.cbk == CB_MUL1);
+}
+int experts_big(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
+                hipStream_t st)
+{
+    const BigPlan p = big_plan(c, R);
+    char* b = (char*)ws;
+    int* G = (int*)(b + p.G);
+    int *gexp = (int*)(b + p.gexp), *goff = (int*)(b + p.goff), *gcnt = (int*)(b + p.gcnt);
+    int *pairmap = (int*)(b + p.pairmap), *prow = (int*)(b + p.prow), *pexp = (int*)(b + p.pexp);
+    uint16_t* xh1 = (uint16_t*)(b + p.xh1);
+    float* part = (float*)(b + p.part);
+    uint16_t* xh2 = (uint16_t*)(b + p.xh2);
+    const uint64_t* tb = (const uint64_t*)tab;
+    prep_big_kernel<<<1, 1024, 0, st>>>(idx, c.itype, R, c.topk, c.E, PG_ROWS, G, gexp, goff, gcnt, pairmap, prow, pexp);
+    int64_t waves = (int64_t)2 * p.P;
+    had_rows_kernel<<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(x, c.xtype, ldx, tb, c.E, 3, 2, p.P, prow, pexp, c.H, xh1);
+    const dim3 g1(c.I / 128, 1, 2 * p.Gmax), g2(c.H / 128, 1, p.Gmax);
+    if (c.cbk == CB_MCG) gemm_kernel<CB_MCG, PG_KT><<<g1, 256, 0, st>>>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, part);
+    else gemm_kernel<CB_MUL1, PG_KT><<<g1, 256, 0, st>>>(xh1, tb, c.E, 0, G, gexp, goff, gcnt, p.Gmax, 2, p.P, c.H, c.I, part);
+    waves = (int64_t)p.P * (c.I / 128);
+    mid_kernel<<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(part, 1, tb, c.E, p.P, c.I, c.act, pexp, xh2, 0);
+    if (c.cbk == CB_MCG) gemm_kernel<CB_MCG, PG_KT><<<g2, 256, 0, st>>>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, part);
+    else gemm_kernel<CB_MUL1, PG_KT><<<g2, 256, 0, st>>>(xh2, tb, c.E, 2, G, gexp, goff, gcnt, p.Gmax, 1, p.P, c.I, c.H, part);
+    waves = (int64_t)R * (c.H / 128);
+    finish_combine_kernel<<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(part, 1, tb, c.E, p.P, c.H, c.topk, pairmap, pexp, w, c.wtype, (const float*)add, (float*)out, R);
+    return launch_status();
+}
+
 // Calls with more rows than one pass takes (64 rows, 1024 pairs) run pass after pass over row ranges: a row's result does not
 // depend on the other rows of a call, so the values are those of one big call.  The passes share the workspace.
 inline int rows_per_pass(const Cfg& c) { const int byp = PMAX / c.topk; return byp < 64 ? byp : 64; }
@@ -367,6 +618,7 @@ int experts_rows(const Cfg& c, const void* x, int64_t ldx, int R, const void* id
     if (R < 1 || c.topk < 1 || c.topk > 64) return -1;
     const int RC = rows_per_pass(c);
     if (R <= RC) return experts(c, x, ldx, R, idx, w, tab, add, out, ws, flags, st);
+    if (!(flags & (4 | 8)) && big_ok(c, R)) return experts_big(c, x, ldx, R, idx, w, tab, add, out, ws, st);     // uniform 4-bit tables: grouped GEMM
     const size_t xsz = c.xtype == X_F32 ? 4 : 2, isz = c.itype ? 8 : 4, wsz = c.wtype ? 2 : 4;
     for (int r0 = 0; r0 < R; r0 += RC) {
         const int n = R - r0 < RC ? R - r0 : RC;
@@ -401,8 +653,10 @@ SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk)
         return plan(c, n).total + (exl3_fused_ok(c, n) ? exl3_fused_ws_bytes(c, n) : 0);
     };
     if (R <= RC) return one(R);
-    const size_t a = one(RC), b = one(R % RC);       // the full passes and the last, shorter one
-    return a == 0 ? 0 : (a > b ? a : b);
+    const size_t a = one(RC), b = one(R % RC);       // the full passes and the last, shorter one (tables with per-expert widths)
+    if (a == 0) return 0;
+    const size_t big = big_ok(c, R) ? big_plan(c, R).total : 0;
+    return a > b ? (a > big ? a : big) : (b > big ? b : big);
 }
 // prepares the workspace once after allocation; calls made with flags bit 0 set then skip their own preparing launch
 SPARK_API int spark_exl3_moe_ws_init(void* ws, size_t bytes, hipStream_t st)

@@ -410,7 +410,12 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
                     bool ok = true;
                     for (int r = wave; r < grp.n; r += FW) {
                         float v0 = 0.f, v1 = 0.f;
-                        if (a.S2 > 1) {
+                        if (a.S2 == 2) {                   // the common split: one word pair, not a round of eight requests
+                            float pl[1], ph[1];
+                            float* pp[1] = {a.part2 + (int64_t)rows[r] * c.H + ncol};
+                            ok = take<LOCAL, 1>(pp, 1, pl, ph) && ok;
+                            v0 += pl[0]; v1 += ph[0];
+                        } else if (a.S2 > 2) {
                             float pl[8], ph[8];
                             float* pp[8];
 #pragma unroll

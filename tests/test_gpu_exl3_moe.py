@@ -195,20 +195,40 @@ def test_glm_three_way_split_widths(ops, oracle):
     assert np.array_equal(out, out2)
 
 
-def test_exl3_moe_prefill_sized_call(ops, oracle):
-    # more rows than one pass takes: the call runs pass after pass over row ranges, the last one short
-    g = synth.rng(490)
-    R, H, I, E, topk = 150, 256, 128, 6, 2
+@pytest.mark.parametrize("R,H,I,E,topk,cbk,act", [(150, 256, 128, 6, 2, 2, 0), (300, 512, 256, 5, 3, 1, 1), (65, 384, 640, 9, 4, 2, 0)])
+def test_exl3_moe_prefill_sized_call(ops, oracle, R, H, I, E, topk, cbk, act):
+    # more than 64 rows: the grouped GEMM over 64-row items (ragged last items, several items per expert)
+    g = synth.rng(490 + R)
     experts = _layer(g, range(E), H, I)
     idx = np.stack([g.permutation(E)[:topk] for _ in range(R)]).astype(np.int32)
     w = g.uniform(0.1, 1.0, (R, topk)).astype(np.float32)
     x = g.standard_normal((R, H)).astype(np.float32)
     add = g.standard_normal((R, H)).astype(np.float32)
     table = ops.ExpertTable(_to_dev(experts), E)
-    out = host(ops.exl3_moe(dev(x), dev(idx), dev(w), table, H, I, add=dev(add)))
-    assert rel_l2(out, oracle.exl3_moe(x, idx, w, experts, E, H, I, 4, 2, 0, add=add)) <= TOL
-    one = host(ops.exl3_moe(dev(x[140:141]), dev(idx[140:141]), dev(w[140:141]), table, H, I, add=dev(add[140:141]), multi_kernel=True))
-    assert np.array_equal(one[0], out[140])                           # a row of the short last pass (several-kernel path), alone
+    out = host(ops.exl3_moe(dev(x), dev(idx), dev(w), table, H, I, codebook=cbk, act=act, add=dev(add)))
+    ref = oracle.exl3_moe(x, idx, w, experts, E, H, I, 4, cbk, act, add=add)
+    assert rel_l2(out, ref) <= TOL, rel_l2(out, ref)
+    out2 = host(ops.exl3_moe(dev(x), dev(idx), dev(w), table, H, I, codebook=cbk, act=act, add=dev(add)))
+    assert np.array_equal(out, out2)                                  # deterministic
+    # a row alone through the decode path: same values within the summation order of the two paths
+    one = host(ops.exl3_moe(dev(x[R - 3:R - 2]), dev(idx[R - 3:R - 2]), dev(w[R - 3:R - 2]), table, H, I, codebook=cbk, act=act, add=dev(add[R - 3:R - 2])))
+    assert rel_l2(one, out[R - 3:R - 2]) <= 3e-4
+
+
+def test_exl3_moe_rows_in_passes_with_per_expert_widths(ops, oracle):
+    # tables with per-expert trellis widths have no grouped GEMM: more than 64 rows run pass after pass over row ranges
+    g = synth.rng(495)
+    R, H, I, E, topk = 70, 256, 128, 4, 2
+    bits = {e: 3 + e % 4 for e in range(E)}
+    experts = {e: synth.exl3_expert(g, H, I, bits[e]) for e in range(E)}
+    table = ops.ExpertTable(_to_dev(experts), E, bits=bits)
+    idx = np.stack([g.permutation(E)[:topk] for _ in range(R)]).astype(np.int32)
+    w = g.uniform(0.1, 1.0, (R, topk)).astype(np.float32)
+    x = g.standard_normal((R, H)).astype(np.float32)
+    out = host(ops.exl3_moe(dev(x), dev(idx), dev(w), table, H, I))
+    for r in (0, 63, 64, R - 1):                                      # rows of the first and of the last pass, each alone
+        one = host(ops.exl3_moe(dev(x[r:r + 1]), dev(idx[r:r + 1]), dev(w[r:r + 1]), table, H, I))
+        assert np.array_equal(one[0], out[r]), r
 
 
 def test_exl3_moe_rejects_bad_shapes(ops):
