@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=640)
     ap.add_argument("--warmup", type=int, default=128)
     ap.add_argument("--batch", type=int, default=1, help="tokens per step of the headline workload (1 or 4)")
-    ap.add_argument("--config", default="c2", choices=["c2", "c3", "c4a", "c4b", "c5"],
+    ap.add_argument("--config", default="c2", choices=["c2", "c3", "c4a", "c4b", "c5", "c2p"],
                     help="headline workload: c2 EXL3 MoE (default, the metric's configuration), c3 MXFP4 MoE, c4a/c4b FP8 dense 7168x4096 / 4096x7168")
     ap.add_argument("--only-headline", action="store_true", help="skip the other configurations' lines")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -114,6 +114,35 @@ class Exl3Layer:
             times.append(time.perf_counter() - t0)
             n += 1
         return float(np.median(times)) * 1e6, n, ref, self.out[n - 1].cpu().numpy()
+
+
+class Exl3Prefill(Exl3Layer):
+    """The config-2 layer at prefill size (2048 tokens): not one of the five configurations, timed next to them because the
+    drop-in takes such calls too (the grouped GEMM of spark_exl3_moe: weights decoded once per 64 rows, fp16 MFMA)."""
+
+    def __init__(self, torch, ops, R, inst, seed=4):
+        super().__init__(torch, ops, R, inst, seed)
+        self.name = f"C2 shape at prefill size: EXL3 4-bit MoE layer (H {self.H}, I {self.I}, {self.E} experts top-{self.TOPK}), {R} tokens"
+        self.flops = 2.0 * R * self.TOPK * 3 * self.H * self.I
+        self.MFMA_PEAK_TFLOPS = 2500.0
+
+    def step(self, i):
+        ops, L = self.ops, self.ops._lib()
+        st = ops._st()
+        k = i % self.inst
+        ops._ck(L.spark_softmax_route(ops._p(self.logits[k]), self.E, self.R, self.E, self.TOPK, ops._p(self.idx[k]), ops._p(self.w[k]), st), "route")
+        ops._ck(L.spark_exl3_moe(ops._p(self.x), 2, self.H, self.R, ops._p(self.idx[k]), 0, ops._p(self.w[k]), 0, ops._p(self.table.tab), None,
+                                 ops._p(self.out[k]), ops._p(self.ws), self.H, self.I, self.E, self.TOPK, 2, 0, 0, st), "exl3_moe")
+
+    dominant = None
+
+    def bytes_per_step(self):
+        idx = self.idx.cpu().numpy()
+        d = np.mean([len(set(idx[k].ravel().tolist())) for k in range(self.inst)])
+        P = self.R * self.TOPK
+        # weights of the distinct experts once + x in, transformed rows out and in (fp16, twice for gate / up), partial sums, y out
+        act = self.R * self.H * 2 + 2 * (2 * P * self.H * 2) + 2 * (2 * P * self.I * 4) + 2 * P * self.I * 2 + 2 * P * self.H * 4 + self.R * self.H * 4
+        return d * self.BYTES_PER_EXPERT + act, float(d)
 
 
 class Mxfp4Layer:
@@ -269,8 +298,9 @@ def line_for(wl, ms):
            "tok_per_s_equiv": round(1e6 / (us * wl.LAYERS) * wl.R, 1), "layers_assumed": wl.LAYERS}
     if hasattr(wl, "flops"):                               # the contraction-sized configuration: matrix-unit rate next to the bandwidth
         tf = wl.flops / (us * 1e-6) / 1e12
-        out.update({"flops": wl.flops, "achieved_TFLOPs": round(tf, 1), "frac_of_fp8_mfma_peak": round(tf / FP8_PEAK_TFLOPS, 4),
-                    "time_at_hbm_peak_us": round(by / (HBM_PEAK_GBS * 1e9) * 1e6, 1), "time_at_mfma_peak_us": round(wl.flops / (FP8_PEAK_TFLOPS * 1e12) * 1e6, 1)})
+        peak = getattr(wl, "MFMA_PEAK_TFLOPS", FP8_PEAK_TFLOPS)      # fp16 operands for the EXL3 GEMM, fp8 for the MXFP4 one
+        out.update({"flops": wl.flops, "achieved_TFLOPs": round(tf, 1), "mfma_peak_TFLOPs": peak, "frac_of_mfma_peak": round(tf / peak, 4),
+                    "time_at_hbm_peak_us": round(by / (HBM_PEAK_GBS * 1e9) * 1e6, 1), "time_at_mfma_peak_us": round(wl.flops / (peak * 1e12) * 1e6, 1)})
     return out
 
 
@@ -302,6 +332,9 @@ def main():
     elif a.config == "c5":
         INST = 4
         wl = Mxfp4Prefill(torch, ops, 2048, INST)
+    elif a.config == "c2p":
+        INST = 4
+        wl = Exl3Prefill(torch, ops, 2048, INST)
     else:
         wl = Fp8Dense(torch, ops, a.batch, INST, *((7168, 4096) if a.config == "c4a" else (4096, 7168)))
     dtype, wset = wl.DTYPE, wl.SET
@@ -330,10 +363,10 @@ def main():
         todo = [lambda: Exl3Layer(torch, ops, 4 if a.batch == 1 else 1, INST)]
         todo += [lambda R=R: Mxfp4Layer(torch, ops, R, INST) for R in (1, 2, 4)]
         todo += [lambda R=R, N=N, K=K: Fp8Dense(torch, ops, R, INST, N, K) for (N, K) in ((7168, 4096), (4096, 7168)) for R in (1, 4)]
-        todo += [lambda: Mxfp4Prefill(torch, ops, 2048, 4)]
+        todo += [lambda: Mxfp4Prefill(torch, ops, 2048, 4), lambda: Exl3Prefill(torch, ops, 2048, 4)]
         for mk in todo:
             w2 = mk()
-            big = isinstance(w2, Mxfp4Prefill)
+            big = isinstance(w2, (Mxfp4Prefill, Exl3Prefill))
             others.append(line_for(w2, time_steps(torch, w2, 32 if big else 256, 8 if big else 64, w2.inst)))
             del w2
             torch.cuda.empty_cache()

@@ -32,32 +32,32 @@ __device__ __forceinline__ void stage_x(const uint16_t* __restrict__ x, int64_t 
 }
 
 // FMT 0: MXFP4 (16 bytes = 32 weights, E8M0 scale per row and 32), 1: FP8 + E8M0 per 32x32, 2: FP8 + fp32 per bs x bs.
-// A wave owns RPW consecutive rows and walks them together, so RPW 16-byte loads per lane are in flight at a time and
-// the activations staged in LDS serve GEMV_WAVES * RPW rows.
-template <int FMT, int M>
+// A wave owns RW consecutive rows and walks them together, so RW 16-byte loads per lane are in flight at a time and
+// the activations staged in LDS serve GEMV_WAVES * RW rows.
+template <int FMT, int M, int RW>
 __global__ __launch_bounds__(64 * GEMV_WAVES) void qgemv_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w, const void* __restrict__ sc,
                                                                 float* __restrict__ y, int m, int n, int k, int xs, int rpg, int bs)
 {
     extern __shared__ uint16_t xl[];                      // [M][k] bf16
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wg_row0 = blockIdx.x * (GEMV_WAVES * RPW);
+    const int wg_row0 = blockIdx.x * (GEMV_WAVES * RW);
     // grouped (block-diagonal) weights read input group row / rpg; a workgroup's rows share the group (rpg % 32 == 0)
     const int64_t xoff = rpg ? (int64_t)(wg_row0 / rpg) * k : 0;
-    const int row0 = wg_row0 + wave * RPW;
+    const int row0 = wg_row0 + wave * RW;
     constexpr int EPP = FMT == 0 ? 32 : 16;               // elements per 16-byte piece
     const int64_t rb = FMT == 0 ? k / 2 : k;              // bytes per weight row
-    float acc[RPW][M];
+    float acc[RW][M];
 #pragma unroll
-    for (int i = 0; i < RPW; ++i)
+    for (int i = 0; i < RW; ++i)
 #pragma unroll
         for (int r = 0; r < M; ++r) acc[i][r] = 0.f;
-    // one step = the lane's 16-byte piece of each of the wave's RPW rows; NS steps are loaded together
-    auto load_steps = [&](auto ns, int c0, uint4 (&p)[UNR][RPW], float (&s)[UNR][RPW]) {
+    // one step = the lane's 16-byte piece of each of the wave's RW rows; NS steps are loaded together
+    auto load_steps = [&](auto ns, int c0, uint4 (&p)[UNR][RW], float (&s)[UNR][RW]) {
 #pragma unroll
         for (int u = 0; u < decltype(ns)::value; ++u) {
             const int c = c0 + u * 64 * EPP;
 #pragma unroll
-            for (int i = 0; i < RPW; ++i) {
+            for (int i = 0; i < RW; ++i) {
                 const int row = row0 + i < n ? row0 + i : n - 1;
                 p[u][i] = ld_stream16(w + (int64_t)row * rb + (FMT == 0 ? c / 2 : c));
                 if (FMT == 0) s[u][i] = e8m0_to_f32(((const uint8_t*)sc)[(int64_t)row * (k >> 5) + (c >> 5)]);
@@ -66,12 +66,12 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void qgemv_kernel(const uint16_t* 
             }
         }
     };
-    auto mul_steps = [&](auto ns, int c0, const uint4 (&p)[UNR][RPW], const float (&s)[UNR][RPW]) {
+    auto mul_steps = [&](auto ns, int c0, const uint4 (&p)[UNR][RW], const float (&s)[UNR][RW]) {
 #pragma unroll
         for (int u = 0; u < decltype(ns)::value; ++u) {
             const int c = c0 + u * 64 * EPP;
 #pragma unroll
-            for (int i = 0; i < RPW; ++i) {
+            for (int i = 0; i < RW; ++i) {
                 const uint32_t pw[4] = {p[u][i].x, p[u][i].y, p[u][i].z, p[u][i].w};
                 bf2 wv[EPP / 2];
 #pragma unroll
@@ -104,8 +104,8 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void qgemv_kernel(const uint16_t* 
             }
         }
     };
-    uint4 p[UNR][RPW];
-    float s[UNR][RPW];
+    uint4 p[UNR][RW];
+    float s[UNR][RW];
     constexpr int BATCH = UNR * 64 * EPP;                 // columns of a full batch of steps
     int c = lane * EPP;
     const bool active = row0 < n;
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void qgemv_kernel(const uint16_t* 
         mul_steps(std::integral_constant<int, 1>{}, c, p, s);
     }
 #pragma unroll
-    for (int i = 0; i < RPW; ++i)
+    for (int i = 0; i < RW; ++i)
 #pragma unroll
         for (int r = 0; r < M; ++r) {
             if (r >= m) break;
@@ -265,6 +265,91 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void bf16_gemv_kernel(const uint16
     }
 }
 
+// FP8 E4M3 weights with one binary32 scale per 128 x 128 block, three or more activation rows: the matrix unit does the
+// multiplies (with one or two rows the dot-product kernel above is as fast and keeps its summation order).  Wave = 16
+// output rows x a quarter of K: a lane's two 16-byte pieces hold 32 neighbouring k of one row, converted to bf16 pairs (exact) and fed as
+// the A operand of v_mfma_f32_16x16x32_bf16, two instructions per piece; the activation rows (padded to 16 columns by
+// repeating the last one) are the B operand from LDS.  Each 128-wide K block accumulates from zero and is added with its
+// scale; the four K quarters of a row tile are summed through LDS in wave order.
+typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
+constexpr int MG_PAD = 8;              // halfs of padding per staged activation row (16-byte reads of 16 rows hit distinct banks)
+__global__ __launch_bounds__(256) void fp8b_mfma_gemv_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w, const float* __restrict__ sc,
+                                                             float* __restrict__ y, int m, int n, int k)
+{
+    extern __shared__ uint16_t xl[];                      // [m][k + MG_PAD] bf16
+    __shared__ float red[4][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, q = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int ks = k / 4, kb0 = wave * ks, nblk = ks / 128, ld = k + MG_PAD, sld = (k + 127) / 128;
+    const int row = min(n0 + c, n - 1);
+    const uint8_t* wp = w + (int64_t)row * k + kb0 + 32 * q;           // a lane's two pieces of a K block are neighbours: four lanes read a whole 128-byte line
+    const float* sp = sc + (int64_t)(n0 / 128) * sld + kb0 / 128;
+    // the first four K blocks are on their way before the activations are staged
+    uint4 p[4][2];
+    float s2[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int b = min(u, nblk - 1);
+        p[u][0] = ld_stream16(wp + b * 128); p[u][1] = ld_stream16(wp + b * 128 + 16);
+        s2[u] = sp[b];
+    }
+    {
+        const int n8 = k / 8;
+        for (int i = threadIdx.x; i < m * n8; i += 256) {
+            const int r = i / n8, cc = (i % n8) * 8;
+            *(uint4*)(xl + r * ld + cc) = *(const uint4*)(x + (int64_t)r * k + cc);
+        }
+    }
+    __syncthreads();
+    const uint16_t* xr = xl + min(c, m - 1) * ld + kb0 + 32 * q;
+    v4f tot = v4f{0.f, 0.f, 0.f, 0.f};
+    auto step = [&](auto uc, int b) {
+        constexpr int u = decltype(uc)::value;
+        v4f cur = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t pw[4] = {p[u][h].x, p[u][h].y, p[u][h].z, p[u][h].w};
+            bf2 wv[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                wv[2 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, false);
+                wv[2 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, true);
+            }
+            const uint4 x0 = *(const uint4*)(xr + b * 128 + h * 16), x1 = *(const uint4*)(xr + b * 128 + h * 16 + 8);
+            bf8v a0, a1, b0, b1;
+            __builtin_memcpy(&a0, &wv[0], 16); __builtin_memcpy(&a1, &wv[4], 16);
+            __builtin_memcpy(&b0, &x0, 16); __builtin_memcpy(&b1, &x1, 16);
+            cur = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, cur, 0, 0, 0);
+            cur = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, cur, 0, 0, 0);
+        }
+        const float sv = s2[u];
+        {                                                 // four blocks ahead, into the registers just used
+            const int bn = min(b + 4, nblk - 1);
+            p[u][0] = ld_stream16(wp + bn * 128); p[u][1] = ld_stream16(wp + bn * 128 + 16);
+            s2[u] = sp[bn];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tot[i] = __builtin_fmaf(cur[i], sv, tot[i]);
+    };
+    for (int b = 0; b < nblk; b += 4) {
+        step(std::integral_constant<int, 0>{}, b);
+        if (b + 1 < nblk) step(std::integral_constant<int, 1>{}, b + 1);
+        if (b + 2 < nblk) step(std::integral_constant<int, 2>{}, b + 2);
+        if (b + 3 < nblk) step(std::integral_constant<int, 3>{}, b + 3);
+    }
+    // D: lane = activation row c, output rows n0 + 4 q + i
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][lane][i] = tot[i];
+    __syncthreads();
+    if (wave == 0 && c < m) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float v = ((red[0][lane][i] + red[1][lane][i]) + red[2][lane][i]) + red[3][lane][i];
+            if (n0 + 4 * q + i < n) y[(int64_t)c * n + n0 + 4 * q + i] = v;
+        }
+    }
+}
+
 constexpr size_t LDS_MAX = 160 * 1024;
 
 template <int FMT>
@@ -272,14 +357,15 @@ int launch_qgemv(const void* x, const void* w, const void* sc, float* y, int m, 
 {
     const size_t sm = (size_t)m * k * 2;
     if (sm > LDS_MAX) return 2;
-    const dim3 g((n + GEMV_WAVES * RPW - 1) / (GEMV_WAVES * RPW)), b(64 * GEMV_WAVES);
-#define QG(MM)                                                                                                                                   \
+    const dim3 b(64 * GEMV_WAVES);
+#define QG(MM, RW)                                                                                                                               \
     do {                                                                                                                                         \
-        static bool attr = hipFuncSetAttribute((const void*)qgemv_kernel<FMT, MM>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX) == hipSuccess; \
+        static bool attr = hipFuncSetAttribute((const void*)qgemv_kernel<FMT, MM, RW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX) == hipSuccess; \
         if (!attr) return 3;                                                                                                                     \
-        qgemv_kernel<FMT, MM><<<g, b, sm, st>>>((const uint16_t*)x, (const uint8_t*)w, sc, y, m, n, k, xs, rpg, bs);                             \
+        const dim3 g((n + GEMV_WAVES * RW - 1) / (GEMV_WAVES * RW));                                                                             \
+        qgemv_kernel<FMT, MM, RW><<<g, b, sm, st>>>((const uint16_t*)x, (const uint8_t*)w, sc, y, m, n, k, xs, rpg, bs);                         \
     } while (0)
-    switch (m) { case 1: QG(1); break; case 2: QG(2); break; case 3: case 4: QG(4); break; default: QG(8); }
+    switch (m) { case 1: QG(1, 4); break; case 2: QG(2, 4); break; case 3: case 4: QG(4, 4); break; default: QG(8, 4); }
 #undef QG
     return launch_status();
 }
@@ -351,6 +437,13 @@ SPARK_API int ds41_fp8_gemv(const void* x, const void* w, const void* ws, float*
 SPARK_API int spark_fp8_block128_gemv(const void* x, const void* w, const float* scales, float* y, int m, int n, int k, hipStream_t st)
 {
     if (m < 1 || m > 8 || n < 1 || k < 16 || k % 16 != 0) return 1;
+    if (m >= 3 && k % 512 == 0 && n % 16 == 0) {          // three or more rows: the matrix unit
+        const size_t sm = (size_t)m * (k + MG_PAD) * 2;
+        if (sm <= 64 * 1024) {
+            fp8b_mfma_gemv_kernel<<<n / 16, 256, sm, st>>>((const uint16_t*)x, (const uint8_t*)w, scales, y, m, n, k);
+            return launch_status();
+        }
+    }
     return launch_qgemv<2>(x, w, scales, y, m, n, k, k, 0, 128, st);
 }
 // reference ds41.cu:251-258: W bf16 [n, k]
