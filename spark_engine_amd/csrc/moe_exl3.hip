@@ -524,6 +524,15 @@ void launch_gemv(const uint16_t* xh, const uint64_t* tab, int E, int slot0, cons
     else gemv_kernel<CBK, 16><<<grid, blk, 0, st>>>(xh, tab, E, slot0, G, gexp, goff, gcnt, Gmax, T, P, K, N, kts, part, vw);
 }
 
+// The single-launch path's region comes first in a workspace and has one size per shape (that of the most rows the path takes),
+// so calls of any size can share a workspace without writing over its idle exchange words.
+inline size_t fused_cap(const Cfg& c)
+{
+    for (int r = 16; r >= 1; --r)
+        if (exl3_fused_ok(c, r)) return exl3_fused_ws_bytes(c, r);
+    return 0;
+}
+
 // flags: bit 0 = the workspace is prepared (once, then only used by these calls);
 //        bit 1 = force the multi-kernel path; bit 2 = mixed trellis widths (table row 9 = bits per expert; multi-kernel path);
 //        bit 3 = every expert has its own intermediate width (table row 10, a multiple of 128 up to I; multi-kernel path)
@@ -535,7 +544,7 @@ int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, co
     const bool varw = (flags & 8) != 0;              // and a row 10 with every expert's intermediate width (reference moe_exl3.cuh:63-67,132-136)
     if (!(flags & 2) && !mixed && !varw && exl3_fused_ok(c, R)) return exl3_fused_launch(c, x, ldx, R, idx, w, tab, add, out, ws, flags & 1, st);
     const Plan p = plan(c, R);
-    char* b = (char*)ws + (exl3_fused_ok(c, R) ? exl3_fused_ws_bytes(c, R) : 0);       // the two paths never share workspace bytes
+    char* b = (char*)ws + fused_cap(c);              // the two paths never share workspace bytes
     int* G = (int*)(b + p.G);
     int *gexp = (int*)(b + p.gexp), *goff = (int*)(b + p.goff), *gcnt = (int*)(b + p.gcnt);
     int *pairmap = (int*)(b + p.pairmap), *prow = (int*)(b + p.prow), *pexp = (int*)(b + p.pexp);
@@ -586,7 +595,7 @@ int experts_big(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx
                 hipStream_t st)
 {
     const BigPlan p = big_plan(c, R);
-    char* b = (char*)ws;
+    char* b = (char*)ws + fused_cap(c);
     int* G = (int*)(b + p.G);
     int *gexp = (int*)(b + p.gexp), *goff = (int*)(b + p.goff), *gcnt = (int*)(b + p.gcnt);
     int *pairmap = (int*)(b + p.pairmap), *prow = (int*)(b + p.prow), *pexp = (int*)(b + p.pexp);
@@ -624,7 +633,7 @@ int experts_rows(const Cfg& c, const void* x, int64_t ldx, int R, const void* id
         const int n = R - r0 < RC ? R - r0 : RC;
         const int rc = experts(c, (const char*)x + (size_t)r0 * ldx * xsz, ldx, n, (const char*)idx + (size_t)r0 * c.topk * isz,
                                (const char*)w + (size_t)r0 * c.topk * wsz, tab, add ? (const float*)add + (size_t)r0 * c.H : nullptr,
-                               (float*)out + (size_t)r0 * c.H, ws, flags & ~1, st);      // a pass of another size leaves other words behind: no "prepared" promise
+                               (float*)out + (size_t)r0 * c.H, ws, flags, st);
         if (rc) return rc;
     }
     return 0;
@@ -648,15 +657,11 @@ SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk)
     const Cfg c{E, topk, H, I, CB_MUL1, 0, 0, 0, 0};
     if (R < 1 || topk < 1 || topk > 64) return 0;
     const int RC = rows_per_pass(c);
-    auto one = [&](int n) -> size_t {
-        if (n < 1 || !cfg_ok(c, n)) return 0;
-        return plan(c, n).total + (exl3_fused_ok(c, n) ? exl3_fused_ws_bytes(c, n) : 0);
-    };
-    if (R <= RC) return one(R);
-    const size_t a = one(RC), b = one(R % RC);       // the full passes and the last, shorter one (tables with per-expert widths)
-    if (a == 0) return 0;
-    const size_t big = big_ok(c, R) ? big_plan(c, R).total : 0;
-    return a > b ? (a > big ? a : big) : (b > big ? b : big);
+    const int n = R < RC ? R : RC;                   // rows of the largest pass
+    if (!cfg_ok(c, n)) return 0;
+    size_t need = plan(c, n).total;
+    if (R > RC && big_ok(c, R)) { const size_t v = big_plan(c, R).total; if (v > need) need = v; }
+    return fused_cap(c) + need;                      // grows with R: a caller may size once for its largest call
 }
 // prepares the workspace once after allocation; calls made with flags bit 0 set then skip their own preparing launch
 SPARK_API int spark_exl3_moe_ws_init(void* ws, size_t bytes, hipStream_t st)

@@ -801,10 +801,18 @@ SPARK_API int spark_mxfp4_prepack(const void* w, const void* s, void* packed, lo
     return launch_status();
 }
 // the single-launch path's workspace follows the several-kernel path's (they never share bytes)
+// The single-launch path's region comes first in a spark_mxfp4_moe* workspace and has one size per shape (that of the most rows the
+// path takes), so calls of any size can share a workspace without writing over its idle exchange words.
+static size_t fused_cap(int H, int I, int topk, int E, int n_shared)
+{
+    for (int r = 8; r >= 1; --r)
+        if (mx_fused_ok(r, H, I, topk, E, n_shared)) return mx_fused_ws_bytes(r, H, I, topk, E, n_shared);
+    return 0;
+}
 SPARK_API size_t spark_mxfp4_moe_ws_bytes(int R, int H, int I, int topk, int E, int n_shared)
 {
     if (!shapes_ok(R, H, I, topk, E, n_shared)) return 0;
-    return ws_layout(R, H, I, topk + n_shared, E + n_shared).total + (mx_fused_ok(R, H, I, topk, E, n_shared) ? mx_fused_ws_bytes(R, H, I, topk, E, n_shared) : 0);
+    return fused_cap(H, I, topk, E, n_shared) + ws_layout(R, H, I, topk + n_shared, E + n_shared).total;     // grows with R
 }
 // prepares a workspace once after allocation (not under stream capture: it also checks workgroup placement, which synchronises);
 // calls of spark_mxfp4_moe_x with flags bit 0 then skip their own preparing launch
@@ -816,7 +824,8 @@ SPARK_API int spark_mxfp4_moe_ws_init(void* ws, size_t bytes, hipStream_t st)
 namespace {
 inline void* fused_ws(void* ws, int R, int H, int I, int topk, int E, int n_shared)
 {
-    return (char*)ws + ws_layout(R, H, I, topk + n_shared, E + n_shared).total;
+    (void)R; (void)H; (void)I; (void)topk; (void)E; (void)n_shared;
+    return ws;                                     // first in the workspace, one size per shape (fused_cap)
 }
 }  // namespace
 // xq [R, H] E4M3 + xs [R, H/32] UE8M0 (act_quant of x); idx int64 / rw f32 [R, topk]; stacked weights of E + n_shared
@@ -831,9 +840,9 @@ SPARK_API int spark_mxfp4_moe_q(const void* xq, const void* xs, int R, const int
         return mx_fused_launch(xq, xs, R, idx, rw, w1, s1, w3, s3, w2, s2, layout, H, I, topk, E, n_shared, add, y, fused_ws(ws, R, H, I, topk, E, n_shared), 0, st);
     if (layout == L_T16)
         return moe_launch<L_T16>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, nullptr, (const uint8_t*)w3, nullptr, (const uint8_t*)w2,
-                                 nullptr, H, I, topk, E, n_shared, add, y, ws, 0, st);
+                                 nullptr, H, I, topk, E, n_shared, add, y, (char*)ws + fused_cap(H, I, topk, E, n_shared), 0, st);
     return moe_launch<L_NATURAL>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3,
-                                 (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, H, I, topk, E, n_shared, add, y, ws, 0, st);
+                                 (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, H, I, topk, E, n_shared, add, y, (char*)ws + fused_cap(H, I, topk, E, n_shared), 0, st);
 }
 extern "C" int ds41_act_quant_fp8(const void* x, void* q, void* s, long long numel, hipStream_t st);
 // x bf16 [R, H]: act_quant per 32 first (scratch xq, xs from the caller: R*H and R*H/32 bytes, used beyond 8 rows), then the experts
@@ -860,9 +869,9 @@ SPARK_API int spark_mxfp4_moe_x(const void* x, const void* xs, int R, const int6
         if (!xs) return 1;
         if (layout == L_T16)
             return moe_launch<L_T16>((const uint8_t*)x, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, nullptr, (const uint8_t*)w3, nullptr,
-                                     (const uint8_t*)w2, nullptr, H, I, topk, E, n_shared, add, y, ws, 0, st);
+                                     (const uint8_t*)w2, nullptr, H, I, topk, E, n_shared, add, y, (char*)ws + fused_cap(H, I, topk, E, n_shared), 0, st);
         return moe_launch<L_NATURAL>((const uint8_t*)x, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3,
-                                     (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, H, I, topk, E, n_shared, add, y, ws, 0, st);
+                                     (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, H, I, topk, E, n_shared, add, y, (char*)ws + fused_cap(H, I, topk, E, n_shared), 0, st);
     }
     if (!mx_fused_ok(R, H, I, topk, E, n_shared)) return 1;
     return mx_fused_launch(x, xs, R, idx, rw, w1, s1, w3, s3, w2, s2, layout, H, I, topk, E, n_shared, add, y, fused_ws(ws, R, H, I, topk, E, n_shared), flags & 1, st);

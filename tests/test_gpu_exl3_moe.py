@@ -231,6 +231,29 @@ def test_exl3_moe_rows_in_passes_with_per_expert_widths(ops, oracle):
         assert np.array_equal(one[0], out[r]), r
 
 
+def test_one_prepared_workspace_serves_calls_of_every_size(ops, oracle):
+    # sized and prepared once for the largest call; decode-sized calls keep their "prepared" promise across larger calls in between
+    g = synth.rng(496)
+    H, I, E, topk = 256, 128, 6, 2
+    experts = _layer(g, range(E), H, I)
+    table = ops.ExpertTable(_to_dev(experts), E)
+    ws = ops.exl3_moe_ws_alloc(100, H, I, E, topk)
+
+    def call(R, seed, clean):
+        gg = synth.rng(seed)
+        idx = np.stack([gg.permutation(E)[:topk] for _ in range(R)]).astype(np.int32)
+        w = gg.uniform(0.1, 1.0, (R, topk)).astype(np.float32)
+        x = gg.standard_normal((R, H)).astype(np.float32)
+        out = host(ops.exl3_moe(dev(x), dev(idx), dev(w), table, H, I, ws=ws, ws_clean=clean))
+        assert rel_l2(out, oracle.exl3_moe(x, idx, w, experts, E, H, I, 4, 2, 0)) <= TOL, R
+        return out
+    first = call(1, 1, True)
+    for R in (4, 20, 64, 100, 16):
+        call(R, 10 + R, True)
+    assert np.array_equal(call(1, 1, True), first)
+    assert int(ws.view(torch.int32)[0].item()) == 0                   # no wait expired
+
+
 def test_exl3_moe_rejects_bad_shapes(ops):
     x = torch.zeros(1, 200, device=DEV)
     with pytest.raises(ops.KernelError):

@@ -113,6 +113,31 @@ def test_grouped_gemm_rows_equal_decode_rows_bitwise(ops, oracle):
         assert np.array_equal(one[0], y[r]), r
 
 
+def test_one_prepared_workspace_serves_calls_of_every_size(ops, oracle):
+    g = synth.rng(214)
+    H, I, E, topk, ns = 1024, 512, 6, 2, 1
+    ws, _, _, _ = _case(g, 1, H, I, E, topk, ns)
+    ex = ops.Mxfp4Experts(*[dev(a) for a in ws], n_shared=ns)
+    wsd = ops.mxfp4_moe_ws_alloc(40, ex, topk)
+
+    def call(R, seed):
+        gg = synth.rng(seed)
+        x = synth.randn_bf16(gg, (R, H))
+        idx = np.stack([gg.permutation(E)[:topk] for _ in range(R)]).astype(np.int64)
+        rw = gg.uniform(0.1, 1.0, (R, topk)).astype(np.float32)
+        if R <= 8:
+            y = host(ops.mxfp4_moe_x(dev_bf16(x), dev(idx), dev(rw), ex, ws=wsd, ws_clean=True))
+        else:
+            y = host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex, ws=wsd))
+        assert rel_l2(y, oracle.mxfp4_moe(x, idx, rw, *ws, n_shared=ns)) <= TOL, R
+        return y
+    first = call(1, 1)
+    for R in (4, 12, 40, 8):
+        call(R, 20 + R)
+    assert np.array_equal(call(1, 1), first)
+    assert int(wsd.view(torch.int32)[0].item()) == 0                  # no wait expired
+
+
 def test_ds41_reference_symbols_tile_layouts(ops, oracle):
     # the reference's own entry points: hidden 5120, weights repacked as kern.rs moe_pack / moe_pack_mx do
     g = synth.rng(213)

@@ -1,0 +1,73 @@
+"""Host-side logic of the C ABI that needs no GPU: workspace sizing, packed sizes, argument checks that return before any launch."""
+import ctypes as C
+
+import pytest
+
+
+@pytest.fixture(scope="module")
+def L():
+    from spark_engine_amd import lib
+    if not lib.SO.exists():
+        pytest.fail(f"{lib.SO} is not built")
+    return lib.load()
+
+
+def test_exl3_workspace_sizes(L):
+    sizes = [L.spark_exl3_moe_ws_bytes(R, 2048, 512, 512, 10) for R in (1, 4, 16, 17, 64, 65, 2048)]
+    assert all(s > 0 for s in sizes)
+    assert sizes == sorted(sizes)                                   # more rows never need less
+    assert sizes[-1] > 2048 * 10 * 2048 * 4                         # the prefill path holds the per-pair outputs
+    assert L.spark_exl3_moe_ws_bytes(1, 2000, 512, 512, 10) == 0    # H not a multiple of 128
+    assert L.spark_exl3_moe_ws_bytes(1, 2048, 500, 512, 10) == 0
+    assert L.spark_exl3_moe_ws_bytes(0, 2048, 512, 512, 10) == 0
+    assert L.spark_exl3_moe_ws_bytes(1, 2048, 512, 512, 0) == 0
+    # the fixed-size entry points size for their models
+    assert L.qwen_moe_ws_bytes(3, 4) == L.spark_exl3_moe_ws_bytes(3, 2560, 640, 512, 10)
+    assert L.glm_moe_ws_bytes(3, 2) == L.spark_exl3_moe_ws_bytes(3, 4096, 1024, 288, 8)
+    assert L.glm_moe3_ws_bytes(3, 2) == L.spark_exl3_moe_ws_bytes(3, 4096, 768, 288, 8)
+
+
+def test_mxfp4_workspace_and_packed_sizes(L):
+    sizes = [L.spark_mxfp4_moe_ws_bytes(R, 4096, 2048, 6, 384, 1) for R in (1, 2, 4, 8, 9, 64, 2048)]
+    assert all(s > 0 for s in sizes) and sizes == sorted(sizes)
+    assert sizes[-1] > 2048 * 7 * 4096 * 4                          # per-pair outputs [P, H] binary32
+    assert L.spark_mxfp4_moe_ws_bytes(1, 4000, 2048, 6, 384, 1) == 0
+    # one 4352-byte record per 16 rows x 512 K
+    assert L.spark_mxfp4_packed_bytes(16, 512) == 4352
+    assert L.spark_mxfp4_packed_bytes(385 * 2048, 4096) == (385 * 2048 // 16) * 8 * 4352
+    assert L.spark_mxfp4_packed_bytes(32, 640) == 2 * 2 * 4352      # a partial K group takes a whole record
+    # the reference-named sizing calls (H fixed at 7168 there)
+    assert L.ds41_moe_mx_ws_bytes(1, 2048, 6, 384) > 0
+    assert L.ds41_moe_ws_bytes(1, 2048, 6, 384) > 0
+
+
+def test_switches(L):
+    L.ds41_moe_mx_set_s2(1)
+    assert L.ds41_moe_mx_get_s2() == 1
+    L.ds41_moe_mx_set_s2(0)
+    assert L.ds41_moe_mx_get_s2() == 0
+    assert L.ds41_fp8_gemv_mx_smem_max() > 0
+
+
+def test_argument_checks_return_before_any_launch(L):
+    null = None
+    # GEMVs: 1 = bad shape (reference ds41.cu:230)
+    assert L.ds41_mxfp4_gemv(null, null, null, null, 9, 16, 64, null) == 1          # more than 8 rows
+    assert L.ds41_mxfp4_gemv(null, null, null, null, 1, 16, 48, null) == 1          # k not a multiple of 32
+    assert L.ds41_fp8_gemv(null, null, null, null, 0, 16, 64, null) == 1
+    assert L.spark_fp8_block128_gemv(null, null, null, null, 1, 16, 24, null) == 1
+    assert L.ds41_act_quant_fp8(null, null, null, 33, null) == 1                    # not whole blocks of 32
+    assert L.ds41_act_quant32(null, null, 0, null) == 0                             # nothing to do
+    # routers
+    assert L.ds41_route(null, null, null, null, 1, 2048, 6, C.c_float(1.0), null) == 1   # too many experts
+    assert L.ds41_route(null, null, null, null, 1, 384, 17, C.c_float(1.0), null) == 1   # top-k above 16
+    # EXL3: -1 dimensions, -4 kmask (reference qwen_exl3.cu:72-128)
+    assert L.spark_exl3_moe(null, 2, 2000, 1, null, 0, null, 0, null, null, null, null, 2000, 512, 512, 10, 2, 0, 0, null) == -1
+    assert L.spark_exl3_moe(null, 2, 2048, 1, null, 0, null, 0, null, null, null, null, 2048, 512, 512, 10, 7, 0, 0, null) == -1   # codebook id
+    assert L.spark_exl3_moe(null, 2, 2049, 1, null, 0, null, 0, null, null, null, null, 2048, 512, 512, 10, 2, 0, 0, null) == -1   # odd row stride
+    assert L.glm_moe_experts(null, 4096, 1, null, null, null, null, null, null, 2, null, 0, null) == -4
+    assert L.glm_moe_experts(null, 4096, 1, null, null, null, null, null, null, 2, null, 1 << 7, null) == -4
+    assert L.glm_moe3_experts(null, 4096, 1, null, null, null, null, null, null, 2, 1 << 2, null) == -4
+    # MXFP4 MoE: 1 = bad shape (reference ds41_mx.cu:1439)
+    assert L.spark_mxfp4_moe_x(null, null, 1, null, null, null, null, null, null, null, null, 0, 4000, 2048, 6, 384, 1, null, null, null, 0, null) == 1
+    assert L.spark_mxfp4_moe_x(null, null, 1, null, null, null, null, null, null, null, null, 9, 4096, 2048, 6, 384, 1, null, null, null, 0, null) == 1   # layout id
