@@ -897,6 +897,9 @@ SPARK_API int ds41_moe_mx_ex(const void* xq, const void* xs, int R, const int64_
                              hipStream_t st)
 {
     if (R < 1 || I % 128 != 0 || E > 384 || topk < 1) return 1;
+    // decode sizes: the whole layer in one launch, straight from the reference's tile layout (same bits as the kernels below)
+    if (!skip_combine && mx_fused_ok(R, DS41_H, I, topk, E, 0))
+        return mx_fused_launch(xq, xs, R, idx, rw, w1, s1, w3, s3, w2, s2, g_s2 ? L_MX8S2 : L_MX8, DS41_H, I, topk, E, 0, add, y, ws, 0, st);
     if (g_s2)                                                  // s1 / s3 / s2 are 2-bit coded scale blobs
         return moe_launch<L_MX8S2>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3,
                                    (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, DS41_H, I, topk, E, 0, add, y, ws, skip_combine, st);
@@ -936,6 +939,9 @@ SPARK_API int ds41_moe(const void* xq, int R, const int64_t* idx, const float* r
                        const void* w2, const void* s2, int I, const float* add, float* y, void* ws, int topk, int E, hipStream_t st)
 {
     if (R < 1 || I % 128 != 0 || E > 384 || topk < 1) return 1;
+    // decode sizes: one launch; the kernel re-encodes the BF16 values itself (act_quant of act-quantised values is exact)
+    if (mx_fused_ok(R, DS41_H, I, topk, E, 0))
+        return mx_fused_launch(xq, nullptr, R, idx, rw, w1, s1, w3, s3, w2, s2, L_PACK8, DS41_H, I, topk, E, 0, add, y, ws, 0, st);
     char* tail = (char*)ws + spark_mxfp4_moe_ws_bytes(R, DS41_H, I, topk, E, 0);
     uint8_t* q = (uint8_t*)tail;
     uint8_t* qs = (uint8_t*)(tail + align256((size_t)R * DS41_H));

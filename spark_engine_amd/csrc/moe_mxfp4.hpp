@@ -57,8 +57,14 @@ __device__ __forceinline__ void load_group(const WMat& m, int e, int row0, int k
             } else {                                        // L_MX8 / L_MX8S2: [rows/8][K/128][8][4 q][4 b][4]
                 const int64_t t8 = row >> 3;
                 const int r8 = (int)(row & 7);
-                const uint32_t* p = (const uint32_t*)(m.w + (t8 * steps + step) * 512 + r8 * 64 + g * 4);
-                c[s] = v4i{(int)p[0], (int)p[4], (int)p[8], (int)p[12]};
+                // the row's 64 bytes of a step are 4 x 4 dwords [q][b] and the lane of K block g needs column b = g: the four lanes
+                // of a row (16 apart) load one q-row each with a 16-byte load and transpose with two rounds of row swaps
+                const uint4 v = ld_stream16(m.w + (t8 * steps + step) * 512 + r8 * 64 + g * 16);
+                const auto a02 = __builtin_amdgcn_permlane32_swap(v.x, v.z, false, false);
+                const auto a13 = __builtin_amdgcn_permlane32_swap(v.y, v.w, false, false);
+                const auto b01 = __builtin_amdgcn_permlane16_swap(a02[0], a13[0], false, false);
+                const auto b23 = __builtin_amdgcn_permlane16_swap(a02[1], a13[1], false, false);
+                c[s] = v4i{(int)b01[0], (int)b01[1], (int)b23[0], (int)b23[1]};
                 if constexpr (LAYOUT == L_MX8) sb = m.s[(t8 * steps + step) * 32 + r8 * 4 + g];
                 else {
                     const uint32_t* d = (const uint32_t*)(m.s + t8 * 16);

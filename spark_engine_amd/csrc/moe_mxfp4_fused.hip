@@ -518,6 +518,7 @@ int mx_fused_launch(const void* x, const void* xs, int R, const int64_t* idx, co
         case L_NATURAL: return quant ? launch<L_NATURAL, true>(a, p, st) : launch<L_NATURAL, false>(a, p, st);
         case L_PACK8: return quant ? launch<L_PACK8, true>(a, p, st) : launch<L_PACK8, false>(a, p, st);
         case L_MX8: return quant ? launch<L_MX8, true>(a, p, st) : launch<L_MX8, false>(a, p, st);
+        case L_MX8S2: return quant ? launch<L_MX8S2, true>(a, p, st) : launch<L_MX8S2, false>(a, p, st);
     }
     return 1;
 }
