@@ -7,8 +7,9 @@
 //       (item, column block) group in launch order is its finisher: it takes the other blocks' partials, finishes gate
 //       and up (Hadamard, svh), applies the activation and the down input transform and hands that block of xh2 to
 //       every down-projection block of the item.
-//   B blocks: (128-column block of H | item, K slice).  Issue and DECODE their down-projection tiles first (they do not
-//       depend on stage 1), then take the item's xh2, dot, finish (Hadamard, svh).  For every token row the block of
+//   B blocks: (128-column block of H | item, K slice of 256).  Issue and DECODE their down-projection tiles first (they do not
+//       depend on stage 1), then take the item's xh2, dot; the last slice's block takes the other slices' sums and finishes
+//       (Hadamard, svh).  For every token row the block of
 //       the row's last item in launch order does the weighted slot-order sum for its 128 columns.
 //
 // Exchange without counters: every exchanged 32-bit word of the workspace is EMPTY (all ones) between uses.  A producer
@@ -24,6 +25,8 @@
 // Only xh2 crosses XCDs, through device-coherent stores / loads.  If the placement check fails, every exchange uses the
 // device-coherent form.
 //
+// Order.  Every A block comes before every B block: a B block that waits for its item must not hold a slot an A block could
+// use (interleaving the two stages item by item was measured 17 % slower at one row and 46 % at four).
 // Progress.  Blocks are dispatched in id order and a block only ever waits for blocks with lower ids (A before B, the
 // finisher is the last block of its group, the summing block belongs to the row's last item), so whatever a block waits
 // for is resident or done.  Waits are bounded: on expiry the block sets an error flag and skips its work, and every
@@ -45,7 +48,8 @@ long long* g_trace = nullptr;
 #endif
 
 constexpr int FW = 4;                 // waves per block
-constexpr int TWB = 4;                // k-tiles per wave of a stage-2 block (all loaded up front): K slice of 512
+constexpr int TWB = 4;                // k-tiles per wave of a stage-2 block (all loaded and decoded up front): K slice of 256.  Eight would
+                                      // spare the split of I = 512 in two slices but need 155 registers: three blocks per CU instead of four
 constexpr int TWMAX = 8;              // most k-tiles per wave of a stage-1 block (4 or 8, chosen per shape)
 constexpr int PF_MAX = 256, RF_MAX = 16;
 constexpr int SPIN_MAX = 200000;
