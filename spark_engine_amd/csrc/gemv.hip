@@ -120,6 +120,12 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void qgemv_kernel(const uint16_t* 
         load_steps(std::integral_constant<int, UNR>{}, c, p, s);
         mul_steps(std::integral_constant<int, UNR>{}, c, p, s);
     }
+    // what is left of the row: the whole-wave steps of it in one batch (up to three), then the ragged end step by step
+    {
+        const int left = (k - c + lane * EPP) / (64 * EPP);         // whole steps left (the same for every lane: c - lane * EPP is uniform)
+        if (left == 3) { load_steps(std::integral_constant<int, 3>{}, c, p, s); mul_steps(std::integral_constant<int, 3>{}, c, p, s); c += 3 * 64 * EPP; }
+        else if (left == 2) { load_steps(std::integral_constant<int, 2>{}, c, p, s); mul_steps(std::integral_constant<int, 2>{}, c, p, s); c += 2 * 64 * EPP; }
+    }
     for (; c < k; c += 64 * EPP) {
         load_steps(std::integral_constant<int, 1>{}, c, p, s);
         mul_steps(std::integral_constant<int, 1>{}, c, p, s);
