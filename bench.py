@@ -33,8 +33,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=640)
     ap.add_argument("--warmup", type=int, default=128)
     ap.add_argument("--batch", type=int, default=1, help="tokens per step of the headline workload (1 or 4)")
-    ap.add_argument("--config", default="c2", choices=["c2", "c3", "c4a", "c4b", "c5", "c2p"],
-                    help="headline workload: c2 EXL3 MoE (default, the metric's configuration), c3 MXFP4 MoE, c4a/c4b FP8 dense 7168x4096 / 4096x7168")
+    ap.add_argument("--config", default="c2", choices=["c2", "c3", "c3w", "c4a", "c4b", "c5", "c2p"],
+                    help="headline workload: c2 EXL3 MoE (default, the metric's configuration), c3 MXFP4 MoE (c3w: the same at hidden width 5120), c4a/c4b FP8 dense 7168x4096 / 4096x7168")
     ap.add_argument("--only-headline", action="store_true", help="skip the other configurations' lines")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", type=int, default=0, metavar="MIB",
@@ -148,7 +148,6 @@ class Exl3Prefill(Exl3Layer):
 class Mxfp4Layer:
     """Config 3: MXFP4 experts, H 4096, I 2048, 384 experts top-6 + 1 shared (sqrt-softplus router)."""
     H, I, E, TOPK, NS, LAYERS = 4096, 2048, 384, 6, 1, 61
-    BYTES_PER_EXPERT = 3 * (4194304 + 262144)
     DTYPE = "fp4 x fp8 (E2M1 weights x E4M3 activations, E8M0 block scales, block-scaled MFMA, fp32 accumulate)"
     SET = "5.1 GB expert set"
 
@@ -157,6 +156,7 @@ class Mxfp4Layer:
         dev = "cuda:0"
         g = torch.Generator(device=dev).manual_seed(seed)
         H, I, ET = self.H, self.I, self.E + self.NS
+        self.BYTES_PER_EXPERT = 3 * (H * I // 2 + H * I // 32)         # codes + one E8M0 byte per 32
         packed = []
         for rows, K in ((I, H), (I, H), (H, I)):
             w = torch.randint(0, 256, (ET, rows, K // 2), dtype=torch.uint8, device=dev, generator=g)
@@ -191,6 +191,13 @@ class Mxfp4Layer:
         idx = self.idx.cpu().numpy()
         d = np.mean([len(set(idx[k].ravel().tolist())) for k in range(self.inst)]) + self.NS
         return d * self.BYTES_PER_EXPERT + self.R * self.H * (2 + 4), float(d)
+
+
+class Mxfp4LayerWide(Mxfp4Layer):
+    """The MXFP4 layer at the hidden width the reference's kernels are compiled for (reference engine-rs/shim/ds41_moe.cu:32, H = 5120):
+    ten 512-wide K groups for the eight waves of a gate/up block."""
+    H = 5120
+    SET = "6.4 GB expert set"
 
 
 class Mxfp4Prefill(Mxfp4Layer):
@@ -329,6 +336,8 @@ def main():
         wl = Exl3Layer(torch, ops, a.batch, INST)
     elif a.config == "c3":
         wl = Mxfp4Layer(torch, ops, a.batch, INST)
+    elif a.config == "c3w":
+        wl = Mxfp4LayerWide(torch, ops, a.batch, INST)
     elif a.config == "c5":
         INST = 4
         wl = Mxfp4Prefill(torch, ops, 2048, INST)

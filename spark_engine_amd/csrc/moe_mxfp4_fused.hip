@@ -77,7 +77,7 @@ __device__ __forceinline__ int pair_expert(const MArgs& a, int p)
 struct Group { int e, n; };      // an item: expert and number of pairs (rows), the pairs ascending in a rows[] array
 
 template <int LAYOUT, bool QUANT, bool LOCAL>
-__global__ __launch_bounds__(NT) void mx_fused_kernel(const MArgs a)
+__global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int sidx[PMAXF], rowsU[RMAX], rowsD[RMAX], comb[RMAX], misc[4], gsel[4];
