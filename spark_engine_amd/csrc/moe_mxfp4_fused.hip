@@ -25,6 +25,7 @@
 //
 // Semantics: reference engine-rs/shim/ds41_moe.cu:1-24, ds41_mx.cu:129-317, engine-rs/src/ds41/kern.rs:1116-1133.
 #include "moe_mxfp4.hpp"
+#include <type_traits>
 
 namespace spk {
 namespace mx {
@@ -127,25 +128,21 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
         // route weight of this lane's item row, requested ahead of the weight rows
         float wgt = 0.f;
         if (c < grp.n) { const int pr = rows[c], k = pr % a.TT; wgt = k < a.topk ? a.rw[(int64_t)(pr / a.TT) * a.topk + k] : 1.0f; }
-        // ---- the first K group of this wave's weight rows, then the activations of its K groups
-        v4i A[4][4];
-        uint32_t sa[4];
-        {
-            const int kg = min(wave, nkg - 1);
-            load_group<LAYOUT>(a.w1, grp.e, j0, kg, lane, A[0], sa[0]);
-            load_group<LAYOUT>(a.w1, grp.e, j0 + 16, kg, lane, A[1], sa[1]);
-            load_group<LAYOUT>(a.w3, grp.e, j0, kg, lane, A[2], sa[2]);
-            load_group<LAYOUT>(a.w3, grp.e, j0 + 16, kg, lane, A[3], sa[3]);
-        }
         unsigned char* xql = extra;                        // [n][H] E4M3 codes of the item's token rows
         unsigned char* xsl = extra + (size_t)a.R * H;      // [n][H / 32] scales
-        if (QUANT) {
-            // act_quant per 32 (reference engine-rs/src/ds41/ops.rs:26-35): 4 lanes x 8 elements per block
+        // activations of this wave's K groups into LDS: act_quant per 32 (reference engine-rs/src/ds41/ops.rs:26-35, 4 lanes x 8
+        // elements per block) of bf16 rows, or (COPY) the caller's codes and scales as they are
+        auto stage_x = [&](auto copy) {
+            constexpr bool COPY = decltype(copy)::value;
             for (int kg = wave; kg < nkg; kg += NW)
                 for (int r = 0; r < grp.n; ++r) {
                     const int k = kg * 512 + lane * 8;
-                    if (k < H) {
-                        const int tok = rows[r] / a.TT;
+                    if (k >= H) continue;
+                    const int tok = rows[r] / a.TT;
+                    if constexpr (COPY) {
+                        *(uint2*)(xql + (size_t)r * H + k) = *(const uint2*)((const uint8_t*)a.x + (int64_t)tok * H + k);
+                        if ((lane & 3) == 0) xsl[(size_t)r * (H >> 5) + (k >> 5)] = a.xs[(int64_t)tok * (H >> 5) + (k >> 5)];
+                    } else {
                         const uint4 raw = *(const uint4*)((const uint16_t*)a.x + (int64_t)tok * H + k);
                         const uint32_t rw4[4] = {raw.x, raw.y, raw.z, raw.w};
                         float v[8];
@@ -165,37 +162,99 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
                         if ((lane & 3) == 0) xsl[(size_t)r * (H >> 5) + (k >> 5)] = (unsigned char)e;
                     }
                 }
-        }
-        TRACE(2);
+        };
         const bool valid = c < grp.n;
         const int rc = valid ? c : 0;
         const int pair = rows[rc];
-        const uint8_t* xr = QUANT ? xql + (size_t)rc * H : (const uint8_t*)a.x + (int64_t)(pair / a.TT) * H;
-        const uint8_t* xsr = QUANT ? xsl + (size_t)rc * (H >> 5) : a.xs + (int64_t)(pair / a.TT) * (H >> 5);
-        v4f acc[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) { acc[t] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(acc[t])); }
-        for (int kg = wave; kg < nkg; kg += NW) {
-            if (kg != wave) {
+        if (nkg <= NW || nkg > NW + 2) {
+            // ---- wave w walks K groups w, w + 8, ... of the four tiles (gate, gate + 16, up, up + 16); normally one K group, loaded
+            // before the wave stages that K group's activations
+            v4i A[4][4];
+            uint32_t sa[4];
+            {
+                const int kg = min(wave, nkg - 1);
                 load_group<LAYOUT>(a.w1, grp.e, j0, kg, lane, A[0], sa[0]);
                 load_group<LAYOUT>(a.w1, grp.e, j0 + 16, kg, lane, A[1], sa[1]);
                 load_group<LAYOUT>(a.w3, grp.e, j0, kg, lane, A[2], sa[2]);
                 load_group<LAYOUT>(a.w3, grp.e, j0 + 16, kg, lane, A[3], sa[3]);
             }
+            if (QUANT) stage_x(std::false_type{});         // read back by this wave only: no barrier
+            TRACE(2);
+            const uint8_t* xr = QUANT ? xql + (size_t)rc * H : (const uint8_t*)a.x + (int64_t)(pair / a.TT) * H;
+            const uint8_t* xsr = QUANT ? xsl + (size_t)rc * (H >> 5) : a.xs + (int64_t)(pair / a.TT) * (H >> 5);
+            v4f acc[4];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const int step = kg * 4 + s;
-                if (step >= steps) break;
-                v8i b; uint32_t sb;
-                load_b(xr, xsr, step, lane, b, sb);
+            for (int t = 0; t < 4; ++t) { acc[t] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(acc[t])); }
+            for (int kg = wave; kg < nkg; kg += NW) {
+                if (kg != wave) {
+                    load_group<LAYOUT>(a.w1, grp.e, j0, kg, lane, A[0], sa[0]);
+                    load_group<LAYOUT>(a.w1, grp.e, j0 + 16, kg, lane, A[1], sa[1]);
+                    load_group<LAYOUT>(a.w3, grp.e, j0, kg, lane, A[2], sa[2]);
+                    load_group<LAYOUT>(a.w3, grp.e, j0 + 16, kg, lane, A[3], sa[3]);
+                }
 #pragma unroll
-                for (int t = 0; t < 4; ++t) acc[t] = mfma_group_step(s, A[t][s], b, acc[t], sa[t], sb);
+                for (int s = 0; s < 4; ++s) {
+                    const int step = kg * 4 + s;
+                    if (step >= steps) break;
+                    v8i b; uint32_t sb;
+                    load_b(xr, xsr, step, lane, b, sb);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) acc[t] = mfma_group_step(s, A[t][s], b, acc[t], sa[t], sb);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) red[wave][t][v][lane] = acc[t][v];
+        } else {
+            // ---- nine or ten K groups (hidden width up to 5120): the (tile, K group) units are dealt so that every wave streams
+            // four or five of them at once.  Wave w owns tile w % 4 and the sums of slots q, q + 2, q + 4, q + 6 (q = w / 4); slot
+            // s is K group s followed, in the same accumulator, by K group s + 8: the order in which a wave that walks K groups
+            // w, w + 8 adds them, so the sums are the same bits.
+            const int t = wave & 3, q = wave >> 2;
+            const bool tail = q + NW < nkg;
+            const WMat& m = t < 2 ? a.w1 : a.w3;
+            const int row0 = j0 + 16 * (t & 1);
+            v4i A[5][4];
+            uint32_t sa[5];
+            load_group<LAYOUT>(m, grp.e, row0, q, lane, A[0], sa[0]);
+            if (tail) load_group<LAYOUT>(m, grp.e, row0, q + NW, lane, A[4], sa[4]);
+            load_group<LAYOUT>(m, grp.e, row0, q + 2, lane, A[1], sa[1]);
+            load_group<LAYOUT>(m, grp.e, row0, q + 4, lane, A[2], sa[2]);
+            load_group<LAYOUT>(m, grp.e, row0, q + 6, lane, A[3], sa[3]);
+            stage_x(std::integral_constant<bool, !QUANT>{});
+            __syncthreads();                               // a wave multiplies K groups that other waves staged
+            TRACE(2);
+            const uint8_t* xr = xql + (size_t)rc * H;
+            const uint8_t* xsr = xsl + (size_t)rc * (H >> 5);
+            auto unit = [&](const v4i (&Au)[4], uint32_t sau, int kg, v4f acc) {
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const int step = kg * 4 + s;
+                    if (step >= steps) break;
+                    v8i b; uint32_t sb;
+                    load_b(xr, xsr, step, lane, b, sb);
+                    acc = mfma_group_step(s, Au[s], b, acc, sau, sb);
+                }
+                return acc;
+            };
+            auto put = [&](int slot, const v4f& acc) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) red[slot][t][v][lane] = acc[v];
+            };
+            v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+            asm volatile("" : "+v"(acc));
+            acc = unit(A[0], sa[0], q, acc);
+            if (tail) acc = unit(A[4], sa[4], q + NW, acc);
+            put(q, acc);
+#pragma unroll
+            for (int j = 1; j < 4; ++j) {
+                acc = v4f{0.f, 0.f, 0.f, 0.f};
+                asm volatile("" : "+v"(acc));
+                acc = unit(A[j], sa[j], q + 2 * j, acc);
+                put(q + 2 * j, acc);
             }
         }
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) red[wave][t][v][lane] = acc[t][v];
         TRACE(3);
         __syncthreads();
         TRACE(4);

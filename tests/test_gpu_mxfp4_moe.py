@@ -64,7 +64,11 @@ def test_moe_zero_codes_give_add(ops):
     assert np.array_equal(host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex, add=dev(add))), add)
 
 
-@pytest.mark.parametrize("R,H,I,E,topk,ns", [(1, 1024, 512, 12, 6, 1), (2, 512, 384, 6, 3, 1), (4, 1024, 256, 5, 2, 2), (8, 512, 256, 4, 2, 0)])
+@pytest.mark.parametrize("R,H,I,E,topk,ns", [(1, 1024, 512, 12, 6, 1), (2, 512, 384, 6, 3, 1), (4, 1024, 256, 5, 2, 2), (8, 512, 256, 4, 2, 0),
+                                             # nine and ten 512-wide K groups for the eight waves of a gate / up block (ten: the reference's
+                                             # hidden width), a ragged last group, and more K groups than the balanced split covers
+                                             (1, 5120, 256, 6, 3, 1), (4, 4608, 128, 5, 2, 0), (2, 4224, 128, 4, 2, 1), (3, 5120, 128, 4, 2, 0),
+                                             (2, 6144, 128, 4, 2, 0)])
 def test_single_launch_equals_several_kernel_path_bitwise(ops, oracle, R, H, I, E, topk, ns):
     # the decode entry runs the whole layer as one launch with the same summation orders as the several-kernel path;
     # a prepared workspace is reused call after call (the exchanged words clear themselves)
