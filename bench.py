@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=640)
     ap.add_argument("--warmup", type=int, default=128)
     ap.add_argument("--batch", type=int, default=1, help="tokens per step of the headline workload (1 or 4)")
-    ap.add_argument("--config", default="c2", choices=["c2", "c3", "c3w", "c4a", "c4b", "c5", "c2p"],
+    ap.add_argument("--config", default="c2", choices=["c2", "c3", "c3w", "c4a", "c4b", "c5", "c5w", "c2p"],
                     help="headline workload: c2 EXL3 MoE (default, the metric's configuration), c3 MXFP4 MoE (c3w: the same at hidden width 5120), c4a/c4b FP8 dense 7168x4096 / 4096x7168")
     ap.add_argument("--only-headline", action="store_true", help="skip the other configurations' lines")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -232,6 +232,12 @@ class Mxfp4Prefill(Mxfp4Layer):
         return d * self.BYTES_PER_EXPERT + act, float(d)
 
 
+class Mxfp4PrefillWide(Mxfp4Prefill):
+    """Config 5 at the hidden width of the reference's kernels (H = 5120, reference engine-rs/shim/ds41_moe.cu:32)."""
+    H = 5120
+    SET = "6.4 GB expert set"
+
+
 class Fp8Dense:
     """Config 4: FP8 E4M3 dense projection with 128x128 FP32 block scales."""
     LAYERS = 1
@@ -341,6 +347,9 @@ def main():
     elif a.config == "c5":
         INST = 4
         wl = Mxfp4Prefill(torch, ops, 2048, INST)
+    elif a.config == "c5w":
+        INST = 4
+        wl = Mxfp4PrefillWide(torch, ops, 2048, INST)
     elif a.config == "c2p":
         INST = 4
         wl = Exl3Prefill(torch, ops, 2048, INST)

@@ -439,6 +439,17 @@ __device__ __forceinline__ v4i ld_a_step(const uint8_t* rec, int s, int lane)
 }
 __device__ __forceinline__ uint32_t ld_a_scales(const uint8_t* rec, int lane) { return *(const uint32_t*)(rec + 4096 + lane * 4); }
 
+// Visit order of the K groups of a gate / up product with more than eight of them: the decode kernels' wave s (of eight) walks K
+// groups s, s + 8 in one accumulator and the eight sums are added in wave order, so visit i is K group kg, `fresh` says that it
+// starts a sum from zero and `last` that its sum is complete.  Up to eight K groups: 0, 1, 2, ..., each its own sum.
+struct KVisit { int kg; bool fresh, last; };
+__device__ __forceinline__ KVisit k_visit(int i, int nkg)
+{
+    const int nl = nkg > UP_WAVES ? nkg - UP_WAVES : 0;    // sums of two K groups: slots 0 .. nl - 1, visited first
+    if (i < 2 * nl) return KVisit{(i >> 1) + UP_WAVES * (i & 1), (i & 1) == 0, (i & 1) != 0};
+    return KVisit{i - nl, true, true};
+}
+
 __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, WMat w1, WMat w3, int H, int I, int TT,
                                                          const int* __restrict__ G, const Item* __restrict__ items, const int* __restrict__ prow,
                                                          const float* __restrict__ pw, uint8_t* __restrict__ hq, uint8_t* __restrict__ hs)
@@ -461,7 +472,7 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
         toks[tid] = prow[pos] / TT;
         wgts[tid] = tid < it.n ? pw[pos] : 0.f;
     }
-    // the wave's weight records: 16 gate and 16 up rows, K group 0 first
+    // the wave's weight records: 16 gate and 16 up rows, the first K group visited (K group 0) first
     const int64_t tile = ((int64_t)it.e * I + f0 + 16 * wave) >> 4;
     const uint8_t* r1 = w1.w + tile * nkg * REC;
     const uint8_t* r3 = w3.w + tile * nkg * REC;
@@ -470,6 +481,7 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
 #pragma unroll
     for (int s = 0; s < 4; ++s) { a[0][s] = ld_a_step(r1, s, lane); a[1][s] = ld_a_step(r3, s, lane); }
     sa[0] = ld_a_scales(r1, lane); sa[1] = ld_a_scales(r3, lane);
+    const int kg1 = k_visit(min(1, nkg - 1), nkg).kg;
     __syncthreads();
     // staging: thread = (row, 32-byte chunk) of a K group; threads 0..31 also carry the row's 16 scale bytes
     const int srow = tid >> 4, sch = tid & 15;
@@ -479,26 +491,30 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
     uint4 x0 = *(const uint4*)xrow, x1 = *(const uint4*)(xrow + 16), xsc = *(const uint4*)xsrow;
     *(uint4*)xdst = x0; *(uint4*)(xdst + 16) = x1;
     if (tid < GT_ROWS) *(uint4*)&xsl[0][tid * 16] = xsc;
-    {
-        const int k1 = min(1, nkg - 1);
-        x0 = *(const uint4*)(xrow + k1 * 512); x1 = *(const uint4*)(xrow + k1 * 512 + 16); xsc = *(const uint4*)(xsrow + k1 * 16);
-    }
+    x0 = *(const uint4*)(xrow + kg1 * 512); x1 = *(const uint4*)(xrow + kg1 * 512 + 16); xsc = *(const uint4*)(xsrow + kg1 * 16);
     __syncthreads();
     v4f tot[2][2];
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) tot[m][rt] = v4f{0.f, 0.f, 0.f, 0.f};
-    for (int kg = 0; kg < nkg; ++kg) {
-        const int buf = kg & 1, kn = min(kg + 1, nkg - 1);
+    v4f cur[2][2];
+    for (int i = 0; i < nkg; ++i) {
+        const KVisit vis = k_visit(i, nkg);
+        const int buf = i & 1, kn = k_visit(min(i + 1, nkg - 1), nkg).kg;
         const uint8_t* n1 = r1 + (int64_t)kn * REC;
         const uint8_t* n3 = r3 + (int64_t)kn * REC;
         const uint32_t san0 = ld_a_scales(n1, lane), san1 = ld_a_scales(n3, lane);
-        v4f cur[2][2];
+        if (vis.fresh) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt) cur[m][rt] = v4f{0.f, 0.f, 0.f, 0.f};
+        }
 #pragma unroll
         for (int m = 0; m < 2; ++m)
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) { cur[m][rt] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(cur[m][rt])); }
+            for (int rt = 0; rt < 2; ++rt) asm volatile("" : "+v"(cur[m][rt]));
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
 #pragma unroll
@@ -515,16 +531,18 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
             a[0][s] = ld_a_step(n1, s, lane);          // the ring slot is free again: the same step of the next K group
             a[1][s] = ld_a_step(n3, s, lane);
         }
+        if (vis.last) {
 #pragma unroll
-        for (int m = 0; m < 2; ++m)
+            for (int m = 0; m < 2; ++m)
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) tot[m][rt] += cur[m][rt];
+                for (int rt = 0; rt < 2; ++rt) tot[m][rt] += cur[m][rt];
+        }
         sa[0] = san0; sa[1] = san1;
         // the next K group of the rows into the other buffer (nobody reads it before the barrier), the one after into registers
         unsigned char* d = xdst + (buf ^ 1) * (GT_ROWS * GT_XS);
         *(uint4*)d = x0; *(uint4*)(d + 16) = x1;
         if (tid < GT_ROWS) *(uint4*)&xsl[buf ^ 1][tid * 16] = xsc;
-        const int k2 = min(kg + 2, nkg - 1);
+        const int k2 = k_visit(min(i + 2, nkg - 1), nkg).kg;
         x0 = *(const uint4*)(xrow + k2 * 512); x1 = *(const uint4*)(xrow + k2 * 512 + 16); xsc = *(const uint4*)(xsrow + k2 * 16);
         __syncthreads();
     }
@@ -703,12 +721,13 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
 // ---------------------------------------------------------------- host side
 // rows per item: 16 for decode sizes, up to 512 rows of an expert beyond (one pass over the expert's weights per item, which
 // stay in registers while the item's rows go by)
-// rows per item: 16 for decode sizes; beyond, 32 for the grouped GEMM (T16 records, K a multiple of 512 that fits the decode
-// kernels' one-K-group-per-wave order) and up to 512 for the other layouts (one pass over the expert's weights per item)
+// rows per item: 16 for decode sizes; beyond, 32 for the grouped GEMM (T16 records, K a multiple of 512, at most sixteen K groups
+// for gate / up and four for down: the orders of summation the decode kernels have) and up to 512 for the other layouts (one
+// pass over the expert's weights per item)
 inline int gr_of(int R, bool gemm) { return R <= 16 ? 16 : gemm ? GT_ROWS : 512; }
 inline bool gemm_ok(int layout, int R, int H, int I)
 {
-    return layout == L_T16 && R > 16 && H % 512 == 0 && I % 512 == 0 && H / 512 <= UP_WAVES && I / 512 <= DN_WAVES && I % GT_FEAT == 0 && H % GT_COLS == 0;
+    return layout == L_T16 && R > 16 && H % 512 == 0 && I % 512 == 0 && H / 512 <= 2 * UP_WAVES && I / 512 <= DN_WAVES && I % GT_FEAT == 0 && H % GT_COLS == 0;
 }
 inline int gmax_of(int R, int TT, int ET, bool gemm)
 {

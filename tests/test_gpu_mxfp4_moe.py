@@ -101,11 +101,13 @@ def test_moe_many_rows_multi_column_groups(ops, oracle):
     assert rel_l2(y, oracle.mxfp4_moe(x, idx, rw, *ws)) <= TOL
 
 
-def test_grouped_gemm_rows_equal_decode_rows_bitwise(ops, oracle):
-    # prefill sizes run as a grouped GEMM over 32-row items: a shared expert (every row), ragged tails, several K groups; every
-    # row must come out with the bits the single-launch decode path gives the row alone
+@pytest.mark.parametrize("H,I", [(2048, 1024), (5120, 512), (6144, 512)])
+def test_grouped_gemm_rows_equal_decode_rows_bitwise(ops, oracle, H, I):
+    # prefill sizes run as a grouped GEMM over 32-row items: a shared expert (every row), ragged tails, several K groups (more than
+    # the eight waves of a decode block at the wider shapes); every row must come out with the bits the single-launch decode path
+    # gives the row alone
     g = synth.rng(213)
-    R, H, I, E, topk, ns = 45, 2048, 1024, 5, 2, 1
+    R, E, topk, ns = 45, 5, 2, 1
     ws, x, idx, rw = _case(g, R, H, I, E, topk, ns)
     ex = ops.Mxfp4Experts(*[dev(a) for a in ws], n_shared=ns)
     xd, idxd, rwd = dev_bf16(x), dev(idx), dev(rw)
