@@ -430,14 +430,67 @@ constexpr int GT_ROWS = 32;            // rows of a GEMM item
 constexpr int GT_XS = 528;             // LDS stride of a staged row: one K group (512 bytes) + 16: conflict-free 16-byte reads down a column
 constexpr int GT_FEAT = 128;           // output features / columns of a block
 
-__device__ __forceinline__ v4i ld_a_step(const uint8_t* rec, int s, int lane)
-{
-    // default cache policy, not a streaming load: an expert's other 32-row items (neighbours in launch order, on the same XCD)
-    // read the same records and find them in the L2 (measured: 1.45 -> 1.25 ms on the 2048-token workload)
-    const uint4 v = *(const uint4*)(rec + s * 1024 + lane * 16);
-    return v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-}
-__device__ __forceinline__ uint32_t ld_a_scales(const uint8_t* rec, int lane) { return *(const uint32_t*)(rec + 4096 + lane * 4); }
+// The A operand of a 16-row tile, one K group (four steps) at a time, for the layouts the grouped GEMM takes.  ATile holds this
+// lane's base addresses; codes(kg, s) is the 16-byte load of step s (default cache policy, not a streaming load: an expert's
+// other 32-row items - neighbours in launch order, on the same XCD - read the same bytes and find them in the L2; measured
+// 1.45 -> 1.25 ms on the 2048-token workload), fix() turns what was loaded into the operand, scales(kg) is the K group's scale
+// dword (byte s = this lane's K block of step s).
+//   T16: records of 4352 bytes, already in operand order.
+//   PACK8 / MX8 (reference engine-rs/src/ds41/kern.rs moe_pack / moe_pack_mx): tiles of 8 rows, [K / 128][8][64 bytes] codes and
+//   [K / 128][8][4] scales.  MX8 keeps a row's 64 bytes as 4 x 4 dwords [q][b] and the lane of K block g needs column b = g: the
+//   four lanes of a row (16 apart) load one q-row each and transpose with two rounds of row swaps.  The scale dword is gathered
+//   the same way: lane (row, g) loads the four block scales of step g and the four lanes transpose 4 x 4 bytes.
+template <int LAYOUT> struct ATile {
+    const uint8_t* w;
+    const uint8_t* sc;
+    static constexpr int KGW = LAYOUT == L_T16 ? REC : 2048, STEPW = LAYOUT == L_T16 ? 1024 : 512, KGS = LAYOUT == L_T16 ? REC : 128;
+    __device__ __forceinline__ ATile(const WMat& m, int64_t row0, int lane)          // row0: first row of the tile in the stacked matrix
+    {
+        const int steps = m.K >> 7;
+        if constexpr (LAYOUT == L_T16) {
+            const uint8_t* rec = m.w + (row0 >> 4) * (int64_t)(steps >> 2) * REC;
+            w = rec + lane * 16; sc = rec + 4096 + lane * 4;
+        } else {
+            const int64_t row = row0 + (lane & 15), t8 = row >> 3;
+            const int r8 = (int)(row & 7), g = lane >> 4;
+            w = m.w + t8 * steps * 512 + r8 * 64 + g * 16;
+            sc = m.s + t8 * steps * 32 + g * 32 + r8 * 4;
+        }
+    }
+    __device__ __forceinline__ v4i codes(int kg, int s) const
+    {
+        const uint4 v = *(const uint4*)(w + (int64_t)kg * KGW + s * STEPW);
+        return v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+    }
+    __device__ __forceinline__ static v4i fix(const v4i& v)
+    {
+        if constexpr (LAYOUT != L_MX8) return v;
+        else {
+            const auto a02 = __builtin_amdgcn_permlane32_swap((uint32_t)v.x, (uint32_t)v.z, false, false);
+            const auto a13 = __builtin_amdgcn_permlane32_swap((uint32_t)v.y, (uint32_t)v.w, false, false);
+            const auto b01 = __builtin_amdgcn_permlane16_swap(a02[0], a13[0], false, false);
+            const auto b23 = __builtin_amdgcn_permlane16_swap(a02[1], a13[1], false, false);
+            return v4i{(int)b01[0], (int)b01[1], (int)b23[0], (int)b23[1]};
+        }
+    }
+    __device__ __forceinline__ uint32_t scales_raw(int kg) const { return *(const uint32_t*)(sc + (int64_t)kg * KGS); }
+    // what scales_raw() loaded -> byte s = the scale of this lane's K block in step s
+    __device__ __forceinline__ static uint32_t scales_fix(uint32_t d, int lane)
+    {
+        if constexpr (LAYOUT == L_T16) return d;
+        else {
+            // lane (row, g) holds M[g][b] = scale(step g, block b) and wants M[s][g] in byte s: a 4 x 4 byte transpose over the four
+            // lanes of the row, 2 x 2 blocks first (partner g ^ 2), then inside the blocks (partner g ^ 1)
+            const int g = lane >> 4;
+            const uint32_t p = __float_as_uint(lane_xor<32>(__uint_as_float(d), lane));
+            // __builtin_amdgcn_perm(hi, lo, sel): result byte i = byte sel[i] of the 8 bytes {hi, lo} (0-3 lo, 4-7 hi)
+            const uint32_t n = (g & 2) ? __builtin_amdgcn_perm(d, p, 0x07060302u) : __builtin_amdgcn_perm(p, d, 0x05040100u);
+            const uint32_t q = __float_as_uint(lane_xor<16>(__uint_as_float(n), lane));
+            return (g & 1) ? __builtin_amdgcn_perm(n, q, 0x07030501u) : __builtin_amdgcn_perm(q, n, 0x06020400u);
+        }
+    }
+};
+constexpr bool gemm_layout(int layout) { return layout == L_T16 || layout == L_PACK8 || layout == L_MX8; }
 
 // Visit order of the K groups of a gate / up product with more than eight of them: the decode kernels' wave s (of eight) walks K
 // groups s, s + 8 in one accumulator and the eight sums are added in wave order, so visit i is K group kg, `fresh` says that it
@@ -450,6 +503,7 @@ __device__ __forceinline__ KVisit k_visit(int i, int nkg)
     return KVisit{i - nl, true, true};
 }
 
+template <int LAYOUT>
 __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, WMat w1, WMat w3, int H, int I, int TT,
                                                          const int* __restrict__ G, const Item* __restrict__ items, const int* __restrict__ prow,
                                                          const float* __restrict__ pw, uint8_t* __restrict__ hq, uint8_t* __restrict__ hs)
@@ -472,15 +526,13 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
         toks[tid] = prow[pos] / TT;
         wgts[tid] = tid < it.n ? pw[pos] : 0.f;
     }
-    // the wave's weight records: 16 gate and 16 up rows, the first K group visited (K group 0) first
-    const int64_t tile = ((int64_t)it.e * I + f0 + 16 * wave) >> 4;
-    const uint8_t* r1 = w1.w + tile * nkg * REC;
-    const uint8_t* r3 = w3.w + tile * nkg * REC;
+    // the wave's weight rows: 16 gate and 16 up rows, the first K group visited (K group 0) first
+    const ATile<LAYOUT> t1(w1, (int64_t)it.e * I + f0 + 16 * wave, lane), t3(w3, (int64_t)it.e * I + f0 + 16 * wave, lane);
     v4i a[2][4];
     uint32_t sa[2];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) { a[0][s] = ld_a_step(r1, s, lane); a[1][s] = ld_a_step(r3, s, lane); }
-    sa[0] = ld_a_scales(r1, lane); sa[1] = ld_a_scales(r3, lane);
+    for (int s = 0; s < 4; ++s) { a[0][s] = t1.codes(0, s); a[1][s] = t3.codes(0, s); }
+    sa[0] = t1.scales_raw(0); sa[1] = t3.scales_raw(0);
     const int kg1 = k_visit(min(1, nkg - 1), nkg).kg;
     __syncthreads();
     // staging: thread = (row, 32-byte chunk) of a K group; threads 0..31 also carry the row's 16 scale bytes
@@ -502,9 +554,8 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
     for (int i = 0; i < nkg; ++i) {
         const KVisit vis = k_visit(i, nkg);
         const int buf = i & 1, kn = k_visit(min(i + 1, nkg - 1), nkg).kg;
-        const uint8_t* n1 = r1 + (int64_t)kn * REC;
-        const uint8_t* n3 = r3 + (int64_t)kn * REC;
-        const uint32_t san0 = ld_a_scales(n1, lane), san1 = ld_a_scales(n3, lane);
+        const uint32_t san0 = t1.scales_raw(kn), san1 = t3.scales_raw(kn);
+        const uint32_t sc0 = ATile<LAYOUT>::scales_fix(sa[0], lane), sc1 = ATile<LAYOUT>::scales_fix(sa[1], lane);
         if (vis.fresh) {
 #pragma unroll
             for (int m = 0; m < 2; ++m)
@@ -517,6 +568,7 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
             for (int rt = 0; rt < 2; ++rt) asm volatile("" : "+v"(cur[m][rt]));
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
+            const v4i a0 = ATile<LAYOUT>::fix(a[0][s]), a1 = ATile<LAYOUT>::fix(a[1][s]);
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
                 if (rt < nrt) {
@@ -524,12 +576,12 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
                     const uint4 lo = *(const uint4*)bp, hi = *(const uint4*)(bp + 64);
                     const v8i b = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
                     const uint32_t sb = *(const uint32_t*)&xsl[buf][(rt * 16 + c) * 16 + s * 4] >> (8 * rg);
-                    cur[0][rt] = mfma_group_step(s, a[0][s], b, cur[0][rt], sa[0], sb);
-                    cur[1][rt] = mfma_group_step(s, a[1][s], b, cur[1][rt], sa[1], sb);
+                    cur[0][rt] = mfma_group_step(s, a0, b, cur[0][rt], sc0, sb);
+                    cur[1][rt] = mfma_group_step(s, a1, b, cur[1][rt], sc1, sb);
                 }
             }
-            a[0][s] = ld_a_step(n1, s, lane);          // the ring slot is free again: the same step of the next K group
-            a[1][s] = ld_a_step(n3, s, lane);
+            a[0][s] = t1.codes(kn, s);                 // the ring slot is free again: the same step of the next K group
+            a[1][s] = t3.codes(kn, s);
         }
         if (vis.last) {
 #pragma unroll
@@ -584,6 +636,7 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
 }
 
 constexpr int GT_COLS = 256;           // output columns of a down-projection block: two 16-column tiles per wave
+template <int LAYOUT>
 __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __restrict__ hq, const uint8_t* __restrict__ hs, WMat w2, int H, int I,
                                                            const int* __restrict__ G, const Item* __restrict__ items, float* __restrict__ out)
 {
@@ -595,14 +648,12 @@ __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __rest
     const int n0 = blockIdx.x * GT_COLS + 32 * wave;
     const int nkg = I >> 9;
     const int nrt = (it.n + 15) >> 4;
-    const int64_t tile = ((int64_t)it.e * H + n0) >> 4;
-    const uint8_t* ra = w2.w + tile * nkg * REC;
-    const uint8_t* rb = ra + (int64_t)nkg * REC;
+    const ATile<LAYOUT> ta(w2, (int64_t)it.e * H + n0, lane), tb(w2, (int64_t)it.e * H + n0 + 16, lane);
     v4i a[2][4];
     uint32_t sa[2];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) { a[0][s] = ld_a_step(ra, s, lane); a[1][s] = ld_a_step(rb, s, lane); }
-    sa[0] = ld_a_scales(ra, lane); sa[1] = ld_a_scales(rb, lane);
+    for (int s = 0; s < 4; ++s) { a[0][s] = ta.codes(0, s); a[1][s] = tb.codes(0, s); }
+    sa[0] = ta.scales_raw(0); sa[1] = tb.scales_raw(0);
     const int srow = tid >> 4, sch = tid & 15;
     const uint8_t* xrow = hq + (int64_t)(it.off + min(srow, it.n - 1)) * I + sch * 32;
     const uint8_t* xsrow = hs + (int64_t)(it.off + min(tid & (GT_ROWS - 1), it.n - 1)) * (I >> 5);
@@ -622,9 +673,8 @@ __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __rest
         for (int rt = 0; rt < 2; ++rt) tot[m][rt] = v4f{0.f, 0.f, 0.f, 0.f};
     for (int kg = 0; kg < nkg; ++kg) {
         const int buf = kg & 1, kn = min(kg + 1, nkg - 1);
-        const uint8_t* na = ra + (int64_t)kn * REC;
-        const uint8_t* nb = rb + (int64_t)kn * REC;
-        const uint32_t san0 = ld_a_scales(na, lane), san1 = ld_a_scales(nb, lane);
+        const uint32_t san0 = ta.scales_raw(kn), san1 = tb.scales_raw(kn);
+        const uint32_t sc0 = ATile<LAYOUT>::scales_fix(sa[0], lane), sc1 = ATile<LAYOUT>::scales_fix(sa[1], lane);
         v4f cur[2][2];
 #pragma unroll
         for (int m = 0; m < 2; ++m)
@@ -632,6 +682,7 @@ __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __rest
             for (int rt = 0; rt < 2; ++rt) { cur[m][rt] = v4f{0.f, 0.f, 0.f, 0.f}; asm volatile("" : "+v"(cur[m][rt])); }
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
+            const v4i a0 = ATile<LAYOUT>::fix(a[0][s]), a1 = ATile<LAYOUT>::fix(a[1][s]);
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
                 if (rt < nrt) {
@@ -639,12 +690,12 @@ __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __rest
                     const uint4 lo = *(const uint4*)bp, hi = *(const uint4*)(bp + 64);
                     const v8i b = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
                     const uint32_t sb = *(const uint32_t*)&xsl[buf][(rt * 16 + c) * 16 + s * 4] >> (8 * rg);
-                    cur[0][rt] = mfma_group_step(s, a[0][s], b, cur[0][rt], sa[0], sb);
-                    cur[1][rt] = mfma_group_step(s, a[1][s], b, cur[1][rt], sa[1], sb);
+                    cur[0][rt] = mfma_group_step(s, a0, b, cur[0][rt], sc0, sb);
+                    cur[1][rt] = mfma_group_step(s, a1, b, cur[1][rt], sc1, sb);
                 }
             }
-            a[0][s] = ld_a_step(na, s, lane);
-            a[1][s] = ld_a_step(nb, s, lane);
+            a[0][s] = ta.codes(kn, s);
+            a[1][s] = tb.codes(kn, s);
         }
 #pragma unroll
         for (int m = 0; m < 2; ++m)
@@ -727,7 +778,7 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
 inline int gr_of(int R, bool gemm) { return R <= 16 ? 16 : gemm ? GT_ROWS : 512; }
 inline bool gemm_ok(int layout, int R, int H, int I)
 {
-    return layout == L_T16 && R > 16 && H % 512 == 0 && I % 512 == 0 && H / 512 <= 2 * UP_WAVES && I / 512 <= DN_WAVES && I % GT_FEAT == 0 && H % GT_COLS == 0;
+    return gemm_layout(layout) && R > 16 && H % 512 == 0 && I % 512 == 0 && H / 512 <= 2 * UP_WAVES && I / 512 <= DN_WAVES && I % GT_FEAT == 0 && H % GT_COLS == 0;
 }
 inline int gmax_of(int R, int TT, int ET, bool gemm)
 {
@@ -773,10 +824,13 @@ int moe_launch(const uint8_t* xq, const uint8_t* xs, int R, const int64_t* idx, 
     float* out = (float*)(base + l.out);
     group_kernel<<<1, 1024, 0, st>>>(idx, rw, R, topk, n_shared, E, GR, G, items, pairmap, prow, pw, G + 4, 64);
     const WMat m1{w1, s1, I, H, (int64_t)ET * I / 8}, m3{w3, s3, I, H, (int64_t)ET * I / 8}, m2{w2, s2, H, I, (int64_t)ET * H / 8};
-    if (gemm) {
-        up_gemm_kernel<<<dim3(I / GT_FEAT, Gm), 512, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
-        down_gemm_kernel<<<dim3(H / GT_COLS, Gm), 512, 0, st>>>(hq, hs, m2, H, I, G, items, out);
-    } else {
+    if constexpr (gemm_layout(LAYOUT)) {
+        if (gemm) {
+            up_gemm_kernel<LAYOUT><<<dim3(I / GT_FEAT, Gm), 512, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
+            down_gemm_kernel<LAYOUT><<<dim3(H / GT_COLS, Gm), 512, 0, st>>>(hq, hs, m2, H, I, G, items, out);
+        }
+    }
+    if (!gemm) {
     if (((H >> 7) + 3) >> 2 <= UP_WAVES) up_res_kernel<LAYOUT><<<dim3(I / 32, Gm), 64 * UP_WAVES, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
     else up_kernel<LAYOUT><<<dim3(I / 32, Gm), 64 * UP_WAVES, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
     if (((I >> 7) + 3) >> 2 <= DN_WAVES) down_res_kernel<LAYOUT><<<dim3(H / 32, Gm), 64 * DN_WAVES, 0, st>>>(hq, hs, m2, H, I, G, items, out);

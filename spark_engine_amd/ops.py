@@ -381,6 +381,8 @@ def ds41_moe_mx(xq, xs, idx, rw, w, I, add=None, skip_combine=False, ws=None):
     """reference kern.rs moe_mx_par / ds41_moe_mx_ex: hidden 5120, weights w = (w1, s1, w3, s3, w2, s2) in the mx tile layout."""
     R = xq.shape[0]
     topk, E = idx.shape[1], w[0].shape[0]
+    if xq.shape[1] != 5120 or xs.shape[1] != 160 or (add is not None and tuple(add.shape) != (R, 5120)):
+        raise ValueError("ds41_moe_mx is compiled for hidden width 5120 (reference ds41_mx.cu:30); use mxfp4_moe for other widths")
     y = torch.empty(R, 5120, dtype=torch.float32, device=xq.device)
     if ws is None:
         ws = torch.empty(_lib().ds41_moe_mx_ws_bytes(R, I, topk, E), dtype=torch.uint8, device=xq.device)
@@ -393,6 +395,8 @@ def ds41_moe(xq_bf16, idx, rw, w, I, add=None):
     """reference kern.rs moe (ds41_moe): weights in the moe_pack tile layout, xq the act-quantized input as bf16."""
     R = xq_bf16.shape[0]
     topk, E = idx.shape[1], w[0].shape[0]
+    if xq_bf16.shape[1] != 5120 or (add is not None and tuple(add.shape) != (R, 5120)):
+        raise ValueError("ds41_moe is compiled for hidden width 5120 (reference ds41_moe.cu:32); use mxfp4_moe for other widths")
     y = torch.empty(R, 5120, dtype=torch.float32, device=xq_bf16.device)
     ws = torch.empty(_lib().ds41_moe_ws_bytes(R, I, topk, E), dtype=torch.uint8, device=xq_bf16.device)
     _ck(_lib().ds41_moe(_p(_dev(xq_bf16)), R, _p(_dev(idx)), _p(_dev(rw)), *[_p(_dev(t)) for t in w], I, _p(add), _p(y), _p(ws), topk, E, _st()), "ds41_moe")

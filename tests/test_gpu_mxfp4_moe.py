@@ -173,6 +173,31 @@ def test_ds41_reference_symbols_tile_layouts(ops, oracle):
     assert np.array_equal(host(y4), host(y))
 
 
+@pytest.mark.parametrize("H,I", [(5120, 512), (5120, 1024)])           # the reference symbols are compiled for hidden width 5120
+def test_ds41_reference_symbols_prefill_sizes(ops, oracle, H, I):
+    # more than 16 rows: the reference's tile layouts go through the grouped GEMM too (their 8-row tiles are read in place), and a
+    # row's bits are those of the record layout's grouped GEMM and of the decode path
+    g = synth.rng(215)
+    R, E, topk = 45, 5, 2
+    ws, x, idx, rw = _case(g, R, H, I, E, topk, 0, smin=119)
+    add = g.standard_normal((R, H)).astype(np.float32)
+    ref = oracle.mxfp4_moe(x, idx, rw, *ws, add=add)
+    d = [dev(a) for a in ws]
+    p1, ps1 = ops.moe_pack(d[0], d[1]); p3, ps3 = ops.moe_pack(d[2], d[3]); p2, ps2 = ops.moe_pack(d[4], d[5])
+    xq, xs = ops.act_quant_fp8(dev_bf16(x))
+    y_mx, _ = ops.ds41_moe_mx(xq, xs, dev(idx), dev(rw), (ops.moe_pack_mx(p1), ps1, ops.moe_pack_mx(p3), ps3, ops.moe_pack_mx(p2), ps2), I, add=dev(add))
+    assert rel_l2(host(y_mx), ref) <= TOL
+    y_p8 = ops.ds41_moe(ops.act_quant(dev_bf16(x)), dev(idx), dev(rw), (p1, ps1, p3, ps3, p2, ps2), I, add=dev(add))
+    assert np.array_equal(host(y_p8), host(y_mx))
+    ex = ops.Mxfp4Experts(*d)
+    y_rec = host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex, add=dev(add)))
+    assert np.array_equal(y_rec, host(y_mx))
+    for r in (0, 33, R - 1):
+        one, _ = ops.ds41_moe_mx(xq[r:r + 1], xs[r:r + 1], dev(idx[r:r + 1]), dev(rw[r:r + 1]),
+                                 (ops.moe_pack_mx(p1), ps1, ops.moe_pack_mx(p3), ps3, ops.moe_pack_mx(p2), ps2), I, add=dev(add[r:r + 1]))
+        assert np.array_equal(host(one)[0], host(y_mx)[r]), r
+
+
 def test_ds41_two_bit_coded_scales(ops, oracle):
     # the reference's lossless 2-bit scale coding (kern.rs moe_scales_s2): nearly constant scales are coded, a tile with a wide
     # row keeps its raw words; the kernels must see the same scale bytes either way

@@ -71,3 +71,19 @@ def test_argument_checks_return_before_any_launch(L):
     # MXFP4 MoE: 1 = bad shape (reference ds41_mx.cu:1439)
     assert L.spark_mxfp4_moe_x(null, null, 1, null, null, null, null, null, null, null, null, 0, 4000, 2048, 6, 384, 1, null, null, null, 0, null) == 1
     assert L.spark_mxfp4_moe_x(null, null, 1, null, null, null, null, null, null, null, null, 9, 4096, 2048, 6, 384, 1, null, null, null, 0, null) == 1   # layout id
+
+
+def test_fixed_width_entry_points_reject_other_widths():
+    # ds41_moe_mx / ds41_moe carry no hidden-width argument (they are compiled for 5120): the wrappers check the operands' shapes
+    # before anything is launched
+    import torch
+    from spark_engine_amd import ops
+    xq = torch.zeros(2, 1024, dtype=torch.uint8)
+    xs = torch.zeros(2, 32, dtype=torch.uint8)
+    idx = torch.zeros(2, 2, dtype=torch.int64)
+    rw = torch.ones(2, 2)
+    w = tuple(torch.zeros(4, 8, dtype=torch.uint8) for _ in range(6))
+    with pytest.raises(ValueError):
+        ops.ds41_moe_mx(xq, xs, idx, rw, w, 128)
+    with pytest.raises(ValueError):
+        ops.ds41_moe(torch.zeros(2, 1024, dtype=torch.bfloat16), idx, rw, w, 128)
