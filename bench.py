@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=640)
     ap.add_argument("--warmup", type=int, default=128)
     ap.add_argument("--batch", type=int, default=1, help="tokens per step of the headline workload (1 or 4)")
-    ap.add_argument("--config", default="c2", choices=["c2", "c3", "c3w", "c4a", "c4b", "c5", "c5w", "c2p"],
+    ap.add_argument("--config", default="c2", choices=["c2", "c2q", "c2g", "c3", "c3w", "c4a", "c4b", "c5", "c5w", "c2p"],
                     help="headline workload: c2 EXL3 MoE (default, the metric's configuration), c3 MXFP4 MoE (c3w: the same at hidden width 5120), c4a/c4b FP8 dense 7168x4096 / 4096x7168")
     ap.add_argument("--only-headline", action="store_true", help="skip the other configurations' lines")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -47,15 +47,16 @@ def parse():
 class Exl3Layer:
     """Config 2: EXL3 4-bit, H 2048, I 512, 512 experts top-10 (mul1 codebook)."""
     H, I, E, TOPK, LAYERS = 2048, 512, 512, 10, 48
-    BYTES_PER_EXPERT = 3 * 524288 + 3 * (2048 + 512) * 2        # trellis + suh/svh (fp16)
     DTYPE = "f16 (4-bit trellis codes decoded to fp16 codebook values, fp32 accumulate)"
     SET = "805 MB expert set"
+    TAG = "C2 qwen-style"
 
     def __init__(self, torch, ops, R, inst, seed=0):
         self.torch, self.ops, self.R, self.inst = torch, ops, R, inst
         dev = "cuda:0"
         g = torch.Generator(device=dev).manual_seed(seed)
         H, I, E = self.H, self.I, self.E
+        self.BYTES_PER_EXPERT = 3 * (H * I // 2) + 3 * (H + I) * 2     # 4-bit trellis + suh / svh (fp16)
 
         def mat(K, N):
             tr = torch.randint(-32768, 32768, (E, K // 16, N // 16, 64), dtype=torch.int16, device=dev, generator=g)
@@ -72,7 +73,7 @@ class Exl3Layer:
         self.w = torch.empty(inst, R, self.TOPK, dtype=torch.float32, device=dev)
         self.out = torch.empty(inst, R, H, dtype=torch.float32, device=dev)
         self.ws = ops.exl3_moe_ws_alloc(R, H, I, E, self.TOPK)
-        self.name = f"C2 qwen-style EXL3 4-bit MoE layer (H {H}, I {I}, {E} experts top-{self.TOPK}), batch {R}"
+        self.name = f"{self.TAG} EXL3 4-bit MoE layer (H {H}, I {I}, {E} experts top-{self.TOPK}), batch {R}"
 
     def step(self, i):
         import ctypes as C
@@ -114,6 +115,20 @@ class Exl3Layer:
             times.append(time.perf_counter() - t0)
             n += 1
         return float(np.median(times)) * 1e6, n, ref, self.out[n - 1].cpu().numpy()
+
+
+class Exl3LayerQwen(Exl3Layer):
+    """The sizes the reference's QwenMoe kernels are compiled for (reference engine-rs/shim/moe_exl3.cuh:24-32)."""
+    H, I, E, TOPK = 2560, 640, 512, 10
+    SET = "1.26 GB expert set"
+    TAG = "reference-sized qwen"
+
+
+class Exl3LayerGlm(Exl3Layer):
+    """The sizes the reference's GlmMoe kernels are compiled for (reference engine-rs/shim/moe_exl3.cuh:35-61)."""
+    H, I, E, TOPK = 4096, 1024, 288, 8
+    SET = "1.81 GB expert set"
+    TAG = "reference-sized glm"
 
 
 class Exl3Prefill(Exl3Layer):
@@ -340,6 +355,10 @@ def main():
     INST = 64
     if a.config == "c2":
         wl = Exl3Layer(torch, ops, a.batch, INST)
+    elif a.config == "c2q":
+        wl = Exl3LayerQwen(torch, ops, a.batch, INST)
+    elif a.config == "c2g":
+        wl = Exl3LayerGlm(torch, ops, a.batch, INST)
     elif a.config == "c3":
         wl = Mxfp4Layer(torch, ops, a.batch, INST)
     elif a.config == "c3w":
@@ -382,6 +401,8 @@ def main():
         todo += [lambda R=R: Mxfp4Layer(torch, ops, R, INST) for R in (1, 2, 4)]
         todo += [lambda R=R, N=N, K=K: Fp8Dense(torch, ops, R, INST, N, K) for (N, K) in ((7168, 4096), (4096, 7168)) for R in (1, 4)]
         todo += [lambda: Mxfp4Prefill(torch, ops, 2048, 4), lambda: Exl3Prefill(torch, ops, 2048, 4)]
+        # the sizes the reference's own kernels are compiled for
+        todo += [lambda: Exl3LayerQwen(torch, ops, 1, INST), lambda: Exl3LayerGlm(torch, ops, 1, INST), lambda: Mxfp4LayerWide(torch, ops, 1, INST)]
         for mk in todo:
             w2 = mk()
             big = isinstance(w2, (Mxfp4Prefill, Exl3Prefill))
