@@ -41,8 +41,10 @@ SPARK_API int qwen_exl3_fold(const void* trellis, const void* suh, const void* s
                              hipStream_t st);
 /* Dense EXL3 linears for M <= 64 rows, trellis widths 3..6 bits, mul1 codebook: y = had128(had128(x * suh) @ inner) * svh in three
  * steps or at once.  xh [M, K] fp16, part [S, M, N] fp32 (S = K slices, summed in order), cnt unused.  qwen_exl3_multi: up to 4
- * linears on the same x (silu bit 0 with n = 2: y[0] = silu(linear 0) * linear 1); its mixed-input form (mg / mn) and side-stream
- * fork (silu bit 2) are not provided (-5).  Replace engine-rs/shim/qwen_exl3.cu:70-206. */
+ * linears on the same x (silu bit 0 with n = 2: y[0] = silu(linear 0) * linear 1); with mg / mn (fp32 [M, 4, K]) the input is
+ * (1/4) sum_s mn[m][s][k] * sigmoid(mg[m][s][k]), also written to xout fp32 [M, K]; silu bits 1 and 2 (separate launches, fork
+ * onto the reference runtime's side stream) are accepted and change nothing here: everything runs on st.
+ * Replace engine-rs/shim/qwen_exl3.cu:70-206. */
 SPARK_API int qwen_exl3_had_in(const void* x, int x_f32, int64_t ldx, const void* suh, void* xh, int M, int K, hipStream_t st);
 SPARK_API int qwen_exl3_had_multi(const void* x, int64_t ldx, int M, int K, int n, const void* const* suh, void* const* xh, hipStream_t st);
 SPARK_API int qwen_exl3_gemv(const void* xh, const void* trellis, void* part, int M, int K, int N, int bits, int S, hipStream_t st);

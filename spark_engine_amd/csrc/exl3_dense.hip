@@ -216,19 +216,40 @@ SPARK_API int qwen_exl3_linear(const void* x, int64_t ldx, const void* suh, cons
     if (rc) return rc;
     return qwen_exl3_finish(part, S, svh, y, 1, ldy, M, N, st);
 }
-// Up to 4 linears on the same x fp32 [M <= 64, K]; silu bit 0 (n = 2): y[0] = silu(linear 0) * linear 1.  The mixed-input form
-// (mg / mn non-null) and the side-stream fork (silu bit 2) belong to the model graph and are not provided: -5.
-// reference qwen_exl3.cu:89-134
+namespace {
+// Mixed input of qwen_exl3_multi: xout[m][k] = (1/4) sum over 4 streams of mn[m][s][k] * sigmoid(mg[m][s][k]), added as
+// (v0 + v1) + (v2 + v3) (reference qwen_exl3.cuh:215-223)
+__global__ __launch_bounds__(256) void mix4_kernel(const float* __restrict__ mg, const float* __restrict__ mn, float* __restrict__ xout, int M, int K)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)M * K) return;
+    const int64_t m = i / K, k = i % K;
+    const float* gr = mg + m * 4 * K + k;
+    const float* nr = mn + m * 4 * K + k;
+    float v[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) v[s] = nr[(int64_t)s * K] / (1.0f + __expf(-gr[(int64_t)s * K]));
+    xout[i] = ((v[0] + v[1]) + (v[2] + v[3])) * 0.25f;
+}
+}  // namespace
+// Up to 4 linears on the same x fp32 [M <= 64, K]; silu bit 0 (n = 2): y[0] = silu(linear 0) * linear 1.  With mg / mn (fp32
+// [M, 4, K]) the input is their gated mean, also written to xout [M, K].  silu bits 1 and 2 (separate launches per linear, fork
+// onto the reference runtime's side stream) choose where the reference runs the work, not what it computes: accepted, everything
+// runs on st.  reference qwen_exl3.cu:89-134
 SPARK_API int qwen_exl3_multi(const void* x, int64_t ldx, const void* mg, const void* mn, void* xout, int M, int K, int n, const void* const* suh,
                               void* const* xh, const void* const* trellis, void* const* part, const int* N, const int* S, const void* const* svh, void* const* y,
                               const int64_t* ldy, const int* bits, int silu, hipStream_t st)
 {
-    (void)xout; (void)xh;
-    if (n < 1 || n > 4 || M > 64 || K % 128) return -1;
-    if (mg || mn || (silu & 4)) return -5;
+    (void)xh;
+    if (n < 1 || n > 4 || M > 64 || M < 1 || K % 128) return -1;
+    if ((mg != nullptr) != (mn != nullptr) || (mg && !xout)) return -1;
     for (int i = 0; i < n; ++i) {
         if (N[i] % 128) return -1;
         if (bits[i] < 3 || bits[i] > 6) return -2;
+    }
+    if (mg) {
+        mix4_kernel<<<(unsigned)(((int64_t)M * K + 255) / 256), 256, 0, st>>>((const float*)mg, (const float*)mn, (float*)xout, M, K);
+        x = xout; ldx = K;
     }
     for (int i = 0; i < n; ++i) {
         const int rc = launch_gemv(1, x, ldx, suh[i], trellis[i], part[i], M, K, N[i], bits[i], S[i], CB_MUL1, st);

@@ -92,20 +92,26 @@ def exl3_linear(x, suh, trellis, svh, S=4):
     return y
 
 
-def exl3_multi(x, linears, S=4, silu=False):
-    """x f32 [M, K]; linears = [(suh, trellis, svh), ...] (at most 4) -> list of y f32 [M, N_i] (one tensor with silu)."""
-    M, K = x.shape
+def exl3_multi(x, linears, S=4, silu=False, mix=None):
+    """x f32 [M, K]; linears = [(suh, trellis, svh), ...] (at most 4) -> list of y f32 [M, N_i] (one tensor with silu).
+    mix = (g, n), both f32 [M, 4, K]: the input is the gated mean of the four streams (x is ignored); returns (ys, xout)."""
+    M, K = (mix[0].shape[0], mix[0].shape[2]) if mix is not None else x.shape
     n = len(linears)
+    if mix is not None:
+        xout = torch.empty(M, K, dtype=torch.float32, device=mix[0].device)
+        x = xout
     Ns = [lin[1].shape[1] * 16 for lin in linears]
     bits = [lin[1].shape[2] // 16 for lin in linears]
     parts = [torch.empty(S, M, N, dtype=torch.float32, device=x.device) for N in Ns]
     ys = [torch.empty(M, N, dtype=torch.float32, device=x.device) for N in Ns]
     vpa = lambda ts: (C.c_void_p * n)(*[t.data_ptr() for t in ts])
     ia = lambda vs: (C.c_int * n)(*vs)
-    _ck(_lib().qwen_exl3_multi(_p(x), x.stride(0), None, None, None, M, K, n, vpa([lin[0] for lin in linears]), None, vpa([lin[1] for lin in linears]),
+    mg, mn, xo = (_p(_dev(mix[0])), _p(_dev(mix[1])), _p(xout)) if mix is not None else (None, None, None)
+    _ck(_lib().qwen_exl3_multi(_p(x), x.stride(0), mg, mn, xo, M, K, n, vpa([lin[0] for lin in linears]), None, vpa([lin[1] for lin in linears]),
                                vpa(parts), ia(Ns), ia([S] * n), vpa([lin[2] for lin in linears]), vpa(ys), (C.c_int64 * n)(*Ns), ia(bits), int(silu), _st()),
         "qwen_exl3_multi")
-    return ys[0] if silu else ys
+    res = ys[0] if (int(silu) & 1) else ys
+    return (res, xout) if mix is not None else res
 
 
 def mxfp4_dequant(w, s):

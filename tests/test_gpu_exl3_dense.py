@@ -72,6 +72,25 @@ def test_multi_and_silu(ops, oracle):
     assert rel_l2(ysilu, a / (1 + np.exp(-a)) * b) <= 1e-3
 
 
+def test_multi_mixed_input(ops, oracle):
+    # the input as the gated mean of four streams (reference qwen_exl3.cuh:200-223): xout against float64 arithmetic, and the
+    # linears on it equal to the linears on xout handed in as x
+    g = synth.rng(511)
+    M, K = 3, 256
+    lins = [synth.exl3_matrix(g, K, N, b) for N, b in ((256, 4), (128, 5))]
+    dl = [(dev_f16(s), dev(t), dev_f16(v)) for t, s, v in lins]
+    mg = g.standard_normal((M, 4, K)).astype(np.float32) * 3
+    mn = g.standard_normal((M, 4, K)).astype(np.float32)
+    ys, xout = ops.exl3_multi(None, dl, S=2, mix=(dev(mg), dev(mn)), silu=4)      # the side-stream bit changes nothing
+    want = (mn.astype(np.float64) / (1 + np.exp(-mg.astype(np.float64)))).sum(1) * 0.25
+    assert np.max(np.abs(host(xout) - want)) <= 1e-5 * np.max(np.abs(want))
+    again = ops.exl3_multi(xout, dl, S=2)
+    for a, b in zip(ys, again):
+        assert np.array_equal(host(a), host(b))
+    for y, (t, s, v) in zip(ys, lins):
+        assert rel_l2(host(y), _reference(oracle, host(xout), t, s, v)[0]) <= 1e-3
+
+
 def test_dense_rejects_bad_arguments(ops):
     x = torch.zeros(2, 200, device=DEV)
     with pytest.raises(ops.KernelError):
