@@ -770,15 +770,14 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
 }
 
 // ---------------------------------------------------------------- host side
-// rows per item: 16 for decode sizes, up to 512 rows of an expert beyond (one pass over the expert's weights per item, which
-// stay in registers while the item's rows go by)
-// rows per item: 16 for decode sizes; beyond, 32 for the grouped GEMM (T16 records, K a multiple of 512, at most sixteen K groups
-// for gate / up and four for down: the orders of summation the decode kernels have) and up to 512 for the other layouts (one
-// pass over the expert's weights per item)
-inline int gr_of(int R, bool gemm) { return R <= 16 ? 16 : gemm ? GT_ROWS : 512; }
+// rows per item: 32 for the grouped GEMM, which takes every call of more than 8 rows that it can (T16 records or the 8-row tile
+// layouts, K a multiple of 512, at most sixteen K groups for gate / up and four for down: the orders of summation the decode
+// kernels have; measured against the kernels below at 9-16 rows: 2-7 % faster on T16 records, 1.8x on the tile layouts at hidden
+// width 5120); otherwise 16 up to 16 rows and up to 512 beyond (one pass over the expert's weights per item)
+inline int gr_of(int R, bool gemm) { return gemm ? GT_ROWS : R <= 16 ? 16 : 512; }
 inline bool gemm_ok(int layout, int R, int H, int I)
 {
-    return gemm_layout(layout) && R > 16 && H % 512 == 0 && I % 512 == 0 && H / 512 <= 2 * UP_WAVES && I / 512 <= DN_WAVES && I % GT_FEAT == 0 && H % GT_COLS == 0;
+    return gemm_layout(layout) && R > 8 && H % 512 == 0 && I % 512 == 0 && H / 512 <= 2 * UP_WAVES && I / 512 <= DN_WAVES && I % GT_FEAT == 0 && H % GT_COLS == 0;
 }
 inline int gmax_of(int R, int TT, int ET, bool gemm)
 {
