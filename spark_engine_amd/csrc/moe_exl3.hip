@@ -528,7 +528,7 @@ void launch_gemv(const uint16_t* xh, const uint64_t* tab, int E, int slot0, cons
 // so calls of any size can share a workspace without writing over its idle exchange words.
 inline size_t fused_cap(const Cfg& c)
 {
-    for (int r = 16; r >= 1; --r)
+    for (int r = 8; r >= 1; --r)
         if (exl3_fused_ok(c, r)) return exl3_fused_ws_bytes(c, r);
     return 0;
 }
@@ -567,7 +567,8 @@ int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, co
     return launch_status();
 }
 
-// ---- prefill: R > 64 rows of a uniform 4-bit table
+// ---- more than 8 rows of a uniform 4-bit table: grouped GEMM over 64-row items (measured against the kernels above on the
+// 512-expert top-10 layer: 9 rows 102 vs 105 us, 16 rows 130 vs 146, 64 rows 272 vs 353)
 struct BigPlan { int P, Gmax; size_t G, gexp, goff, gcnt, pairmap, prow, pexp, xh1, part, xh2, total; };
 inline BigPlan big_plan(const Cfg& c, int R)
 {
@@ -588,7 +589,7 @@ inline BigPlan big_plan(const Cfg& c, int R)
 }
 inline bool big_ok(const Cfg& c, int R)
 {
-    return R > 64 && c.E >= 1 && c.E <= EBIG && c.topk >= 1 && c.topk <= 64 && (int64_t)R * c.topk < (1ll << 24) && c.H >= 128 && c.I >= 128 &&
+    return R > 8 && c.E >= 1 && c.E <= EBIG && c.topk >= 1 && c.topk <= 64 && (int64_t)R * c.topk < (1ll << 24) && c.H >= 128 && c.I >= 128 &&
            c.H % 128 == 0 && c.I % 128 == 0 && (c.cbk == CB_MCG || c.cbk == CB_MUL1);
 }
 int experts_big(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
@@ -618,7 +619,8 @@ int experts_big(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx
     return launch_status();
 }
 
-// Calls with more rows than one pass takes (64 rows, 1024 pairs) run pass after pass over row ranges: a row's result does not
+// Calls the grouped GEMM does not take (tables with per-expert trellis or intermediate widths, the forced several-kernel
+// path) with more rows than one pass takes (64 rows, 1024 pairs) run pass after pass over row ranges: a row's result does not
 // depend on the other rows of a call, so the values are those of one big call.  The passes share the workspace.
 inline int rows_per_pass(const Cfg& c) { const int byp = PMAX / c.topk; return byp < 64 ? byp : 64; }
 int experts_rows(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, const void* w, const void* tab, const void* add, void* out, void* ws,
@@ -626,8 +628,8 @@ int experts_rows(const Cfg& c, const void* x, int64_t ldx, int R, const void* id
 {
     if (R < 1 || c.topk < 1 || c.topk > 64) return -1;
     const int RC = rows_per_pass(c);
+    if (!(flags & (2 | 4 | 8)) && big_ok(c, R)) return experts_big(c, x, ldx, R, idx, w, tab, add, out, ws, st);     // uniform 4-bit tables: grouped GEMM
     if (R <= RC) return experts(c, x, ldx, R, idx, w, tab, add, out, ws, flags, st);
-    if (!(flags & (4 | 8)) && big_ok(c, R)) return experts_big(c, x, ldx, R, idx, w, tab, add, out, ws, st);     // uniform 4-bit tables: grouped GEMM
     const size_t xsz = c.xtype == X_F32 ? 4 : 2, isz = c.itype ? 8 : 4, wsz = c.wtype ? 2 : 4;
     for (int r0 = 0; r0 < R; r0 += RC) {
         const int n = R - r0 < RC ? R - r0 : RC;
@@ -649,9 +651,9 @@ const Cfg GLM3{288, 8, 4096, 768, CB_MCG, 1, X_F16, 1, 1};        // TP3: expert
 
 // Runtime-sized entry (no reference counterpart symbol): x [R, H] of xtype (0 f32, 1 f16, 2 bf16), row stride ldx;
 // idx [R, topk] int32 (itype 0) or int64 (1); w [R, topk] f32 (wtype 0) or f16 (1); tab u64 [9][E]; codebook 2 = mul1,
-// 1 = mcg; act 0 = silu(g) u, 1 = clamped; add / out f32 [R, H].  Any R: more than 64 rows (1024 pairs) run as several passes.
+// 1 = mcg; act 0 = silu(g) u, 1 = clamped; add / out f32 [R, H].  Any R: up to 8 rows in one launch, more as a grouped GEMM (or, for tables the GEMM does not take, as passes of 64 rows).
 // flags bit 0: the workspace was zeroed by spark_exl3_moe_ws_init and only used by this entry since (saves a launch);
-// bit 1: use the multi-kernel path even where the single-launch path applies.
+// bit 1: use the several-kernel path even where the single-launch path or the grouped GEMM applies.
 SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk)
 {
     const Cfg c{E, topk, H, I, CB_MUL1, 0, 0, 0, 0};
@@ -660,7 +662,7 @@ SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk)
     const int n = R < RC ? R : RC;                   // rows of the largest pass
     if (!cfg_ok(c, n)) return 0;
     size_t need = plan(c, n).total;
-    if (R > RC && big_ok(c, R)) { const size_t v = big_plan(c, R).total; if (v > need) need = v; }
+    if (big_ok(c, R)) { const size_t v = big_plan(c, R).total; if (v > need) need = v; }
     return fused_cap(c) + need;                      // grows with R: a caller may size once for its largest call
 }
 // prepares the workspace once after allocation; calls made with flags bit 0 set then skip their own preparing launch

@@ -25,7 +25,7 @@ __device__ __forceinline__ float exl3_act(int act, float a, float u)
     return a / (1.0f + __expf(-a)) * u;
 }
 
-// the single-launch decode path (moe_exl3_fused.hip): usable for R <= 16 rows and R * topk <= 256 pairs
+// the single-launch decode path (moe_exl3_fused.hip): usable for R <= 8 rows and R * topk <= 128 pairs
 bool exl3_fused_ok(const Exl3Cfg& c, int R);
 size_t exl3_fused_ws_bytes(const Exl3Cfg& c, int R);
 // The exchanged words of ws must be in their idle state on entry (they are again when the call has finished): clean = 0

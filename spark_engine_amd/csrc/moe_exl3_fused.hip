@@ -1,4 +1,4 @@
-// Routed EXL3 experts in ONE launch for decode-sized calls (R <= 16 rows, R * topk <= 256 pairs).
+// Routed EXL3 experts in ONE launch for decode-sized calls (R <= 8 rows, R * topk <= 128 pairs).
 //
 // The multi-kernel path (moe_exl3.hip) needs seven dependent launches for a layer that moves 16 MB: launch gaps and the
 // chain of cold first loads cost far more than the weight stream.  Here one grid holds both weight streams:
@@ -51,7 +51,7 @@ constexpr int FW = 4;                 // waves per block
 constexpr int TWB = 4;                // k-tiles per wave of a stage-2 block (all loaded and decoded up front): K slice of 256.  Eight would
                                       // spare the split of I = 512 in two slices but need 155 registers: three blocks per CU instead of four
 constexpr int TWMAX = 8;              // most k-tiles per wave of a stage-1 block (4 or 8, chosen per shape)
-constexpr int PF_MAX = 256, RF_MAX = 16;
+constexpr int PF_MAX = 128, RF_MAX = 8;            // more rows go through the grouped GEMM (faster from 9 rows on)
 constexpr int SPIN_MAX = 200000;
 constexpr int EMAX_F = 1024;           // most experts of a layer on this path
 constexpr int SMAX = 8;               // K slices per product (K <= 4096)
@@ -512,8 +512,7 @@ void launch3(const FArgs& a, int maxrows, hipStream_t st)
     if (maxrows <= 1) fused_kernel<CBK, 1, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
     else if (maxrows <= 2) fused_kernel<CBK, 2, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
     else if (maxrows <= 4) fused_kernel<CBK, 4, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
-    else if (maxrows <= 8) fused_kernel<CBK, 8, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
-    else fused_kernel<CBK, 16, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
+    else fused_kernel<CBK, 8, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
 }
 template <int CBK>
 void launch(const FArgs& a, int twa, int maxrows, hipStream_t st)
