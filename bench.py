@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=640)
     ap.add_argument("--warmup", type=int, default=128)
     ap.add_argument("--batch", type=int, default=1, help="tokens per step of the headline workload (1 or 4)")
-    ap.add_argument("--config", default="c2", choices=["c2", "c2q", "c2g", "c3", "c3w", "c4a", "c4b", "c5", "c5w", "c2p"],
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c2q", "c2g", "c3", "c3w", "c4a", "c4b", "c5", "c5w", "c2p"],
                     help="headline workload: c2 EXL3 MoE (default, the metric's configuration), c3 MXFP4 MoE (c3w: the same at hidden width 5120), c4a/c4b FP8 dense 7168x4096 / 4096x7168")
     ap.add_argument("--only-headline", action="store_true", help="skip the other configurations' lines")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -279,6 +279,32 @@ class Fp8Dense:
         return self.N * self.K + self.s[0].numel() * 4 + self.R * self.K * 2 + self.R * self.N * 4, 1.0
 
 
+class Mxfp4Dense:
+    """Config 1: MXFP4 dense GEMV 2048 x 2048, one row (the reference's own CPU-runnable case, reference ds41.cu:75-110, 236)."""
+    LAYERS = 1
+    DTYPE = "fp4 x bf16 (E2M1 weights, E8M0 block scales, fp32 accumulate)"
+    SET = "rotating over 256 weight copies (570 MB)"
+
+    def __init__(self, torch, ops, R, inst, N=2048, K=2048, seed=6):
+        self.torch, self.ops, self.R, self.inst, self.N, self.K = torch, ops, R, inst, N, K
+        dev = "cuda:0"
+        g = torch.Generator(device=dev).manual_seed(seed)
+        self.ncopy = inst
+        self.w = torch.randint(0, 256, (self.ncopy, N, K // 2), dtype=torch.uint8, device=dev, generator=g)
+        self.s = torch.randint(117, 128, (self.ncopy, N, K // 32), dtype=torch.uint8, device=dev, generator=g)
+        self.x = torch.randn(R, K, device=dev, generator=g).to(torch.bfloat16)
+        self.y = torch.empty(R, N, dtype=torch.float32, device=dev)
+        self.name = f"C1 MXFP4 dense GEMV {N}x{K}, batch {R}"
+
+    def step(self, i):
+        ops, k = self.ops, i % self.ncopy
+        ops._ck(ops._lib().ds41_mxfp4_gemv(ops._p(self.x), ops._p(self.w[k]), ops._p(self.s[k]), ops._p(self.y), self.R, self.N, self.K, ops._st()),
+                "ds41_mxfp4_gemv")
+
+    def bytes_per_step(self):
+        return self.N * self.K // 2 + self.N * self.K // 32 + self.R * self.K * 2 + self.R * self.N * 4, 1.0
+
+
 # ---------------------------------------------------------------------------------------------- timing
 
 def time_steps(torch, wl, steps, warmup, inst, fn=None):
@@ -355,6 +381,9 @@ def main():
     INST = 64
     if a.config == "c2":
         wl = Exl3Layer(torch, ops, a.batch, INST)
+    elif a.config == "c1":
+        INST = 256                                      # 2.2 MB per matrix: 256 copies so that a graph's reads exceed every cache
+        wl = Mxfp4Dense(torch, ops, a.batch, INST)
     elif a.config == "c2q":
         wl = Exl3LayerQwen(torch, ops, a.batch, INST)
     elif a.config == "c2g":
@@ -400,6 +429,7 @@ def main():
         todo = [lambda: Exl3Layer(torch, ops, 4 if a.batch == 1 else 1, INST)]
         todo += [lambda R=R: Mxfp4Layer(torch, ops, R, INST) for R in (1, 2, 4)]
         todo += [lambda R=R, N=N, K=K: Fp8Dense(torch, ops, R, INST, N, K) for (N, K) in ((7168, 4096), (4096, 7168)) for R in (1, 4)]
+        todo += [lambda: Mxfp4Dense(torch, ops, 1, 256)]
         todo += [lambda: Mxfp4Prefill(torch, ops, 2048, 4), lambda: Exl3Prefill(torch, ops, 2048, 4)]
         # the sizes the reference's own kernels are compiled for
         todo += [lambda: Exl3LayerQwen(torch, ops, 1, INST), lambda: Exl3LayerGlm(torch, ops, 1, INST), lambda: Mxfp4LayerWide(torch, ops, 1, INST)]
