@@ -271,39 +271,59 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void bf16_gemv_kernel(const uint16
     }
 }
 
-// FP8 E4M3 weights with one binary32 scale per 128 x 128 block, three or more activation rows: the matrix unit does the
-// multiplies (with one or two rows the dot-product kernel above is as fast and keeps its summation order).  Wave = 16
-// output rows x a quarter of K: a lane's two 16-byte pieces hold 32 neighbouring k of one row, converted to bf16 pairs (exact) and fed as
-// the A operand of v_mfma_f32_16x16x32_bf16, two instructions per piece; the activation rows (padded to 16 columns by
-// repeating the last one) are the B operand from LDS.  Each 128-wide K block accumulates from zero and is added with its
-// scale; the four K quarters of a row tile are summed through LDS in wave order.
+// Three or more activation rows: the matrix unit does the multiplies (with one or two rows the dot-product kernel above is as
+// fast and keeps its summation order).  Wave = 16 output rows x a quarter of K: a lane's piece of a 128-wide K block holds 32
+// neighbouring k of one row (two 16-byte loads of E4M3, one of E2M1), converted to bf16 pairs (exact) and fed as the A operand of
+// v_mfma_f32_16x16x32_bf16, one instruction per 8 weights; the activation rows (padded to 16 columns by repeating the last one)
+// are the B operand from LDS.  Each 128-wide K block accumulates from zero and is added with a binary32 factor: the block's scale
+// (FMT 2), or for the E8M0 formats, whose scale belongs to the lane's 32 k, the largest scale of the wave's 64 pieces - the
+// convert applies every piece's scale relative to that one (a power of two at most 1: never an overflow, and what underflows is
+// below 2^-100 of the block's largest term).  The four K quarters of a row tile are summed through LDS in wave order.
 typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
 constexpr int MG_PAD = 8;              // halfs of padding per staged activation row (16-byte reads of 16 rows hit distinct banks)
-__global__ __launch_bounds__(256) void fp8b_mfma_gemv_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w, const float* __restrict__ sc,
-                                                             float* __restrict__ y, int m, int n, int k)
+__device__ __forceinline__ int wave_max_i(int v)
+{
+    const int lane = threadIdx.x & 63;                    // lane_xor only moves bits: no floating-point operation touches them
+    v = max(v, __float_as_int(lane_xor<32>(__int_as_float(v), lane))); v = max(v, __float_as_int(lane_xor<16>(__int_as_float(v), lane)));
+    v = max(v, __float_as_int(lane_xor<8>(__int_as_float(v), lane))); v = max(v, __float_as_int(lane_xor<4>(__int_as_float(v), lane)));
+    v = max(v, __float_as_int(lane_xor<2>(__int_as_float(v), lane))); v = max(v, __float_as_int(lane_xor<1>(__int_as_float(v), lane)));
+    return v;
+}
+template <int FMT>
+__global__ __launch_bounds__(256) void q_mfma_gemv_kernel(const uint16_t* __restrict__ x, int64_t xs, const uint8_t* __restrict__ w, const void* __restrict__ scv,
+                                                          float* __restrict__ y, int m, int n, int k)
 {
     extern __shared__ uint16_t xl[];                      // [m][k + MG_PAD] bf16
     __shared__ float red[4][64][4];
+    constexpr int NP = FMT == 0 ? 1 : 2;                  // 16-byte loads per piece
+    constexpr int BPB = FMT == 0 ? 64 : 128;              // weight bytes of a row per 128-wide K block
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, q = lane >> 4;
     const int n0 = blockIdx.x * 16;
     const int ks = k / 4, kb0 = wave * ks, nblk = ks / 128, ld = k + MG_PAD, sld = (k + 127) / 128;
     const int row = min(n0 + c, n - 1);
-    const uint8_t* wp = w + (int64_t)row * k + kb0 + 32 * q;           // a lane's two pieces of a K block are neighbours: four lanes read a whole 128-byte line
-    const float* sp = sc + (int64_t)(n0 / 128) * sld + kb0 / 128;
+    // a lane's pieces of a K block are neighbours: four lanes read a whole line of the row
+    const uint8_t* wp = w + (FMT == 0 ? (int64_t)row * (k / 2) + (kb0 + 32 * q) / 2 : (int64_t)row * k + kb0 + 32 * q);
+    const float* spf = (const float*)scv + (int64_t)(n0 / 128) * sld + kb0 / 128;                                  // FMT 2: one per block
+    const uint8_t* spb = (const uint8_t*)scv + (int64_t)(FMT == 1 ? row / 32 : row) * (k / 32) + kb0 / 32 + q;     // E8M0: one per piece
     // the first four K blocks are on their way before the activations are staged
-    uint4 p[4][2];
+    uint4 p[4][NP];
     float s2[4];
+    uint32_t sb[4];
+    auto fetch = [&](auto uc, int b) {
+        constexpr int u = decltype(uc)::value;
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int b = min(u, nblk - 1);
-        p[u][0] = ld_stream16(wp + b * 128); p[u][1] = ld_stream16(wp + b * 128 + 16);
-        s2[u] = sp[b];
-    }
+        for (int h = 0; h < NP; ++h) p[u][h] = ld_stream16(wp + b * BPB + h * 16);
+        if constexpr (FMT == 2) s2[u] = spf[b]; else sb[u] = spb[b * 4];
+    };
+    fetch(std::integral_constant<int, 0>{}, 0);
+    fetch(std::integral_constant<int, 1>{}, min(1, nblk - 1));
+    fetch(std::integral_constant<int, 2>{}, min(2, nblk - 1));
+    fetch(std::integral_constant<int, 3>{}, min(3, nblk - 1));
     {
         const int n8 = k / 8;
         for (int i = threadIdx.x; i < m * n8; i += 256) {
             const int r = i / n8, cc = (i % n8) * 8;
-            *(uint4*)(xl + r * ld + cc) = *(const uint4*)(x + (int64_t)r * k + cc);
+            *(uint4*)(xl + r * ld + cc) = *(const uint4*)(x + (int64_t)r * xs + cc);
         }
     }
     __syncthreads();
@@ -312,14 +332,33 @@ __global__ __launch_bounds__(256) void fp8b_mfma_gemv_kernel(const uint16_t* __r
     auto step = [&](auto uc, int b) {
         constexpr int u = decltype(uc)::value;
         v4f cur = v4f{0.f, 0.f, 0.f, 0.f};
+        float cs = 1.0f, sv;
+        if constexpr (FMT == 2) sv = s2[u];
+        else {
+            const int top = wave_max_i((int)sb[u]);
+            cs = __uint_as_float((uint32_t)max((int)sb[u] - top + 127, 0) << 23);
+            sv = e8m0_to_f32((uint32_t)top);
+        }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const uint32_t pw[4] = {p[u][h].x, p[u][h].y, p[u][h].z, p[u][h].w};
             bf2 wv[8];
+            if constexpr (FMT == 0) {
+                const uint32_t pw[2] = {h ? p[u][0].z : p[u][0].x, h ? p[u][0].w : p[u][0].y};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                wv[2 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, false);
-                wv[2 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, true);
+                for (int j = 0; j < 2; ++j) {
+                    wv[4 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], cs, 0);
+                    wv[4 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], cs, 1);
+                    wv[4 * j + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], cs, 2);
+                    wv[4 * j + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], cs, 3);
+                }
+            } else {
+                const uint4 pv = p[u][NP - 1 < h ? NP - 1 : h];
+                const uint32_t pw[4] = {pv.x, pv.y, pv.z, pv.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    wv[2 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], cs, false);
+                    wv[2 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], cs, true);
+                }
             }
             const uint4 x0 = *(const uint4*)(xr + b * 128 + h * 16), x1 = *(const uint4*)(xr + b * 128 + h * 16 + 8);
             bf8v a0, a1, b0, b1;
@@ -328,12 +367,7 @@ __global__ __launch_bounds__(256) void fp8b_mfma_gemv_kernel(const uint16_t* __r
             cur = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, cur, 0, 0, 0);
             cur = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, cur, 0, 0, 0);
         }
-        const float sv = s2[u];
-        {                                                 // four blocks ahead, into the registers just used
-            const int bn = min(b + 4, nblk - 1);
-            p[u][0] = ld_stream16(wp + bn * 128); p[u][1] = ld_stream16(wp + bn * 128 + 16);
-            s2[u] = sp[bn];
-        }
+        fetch(uc, min(b + 4, nblk - 1));                  // four blocks ahead, into the registers just used
 #pragma unroll
         for (int i = 0; i < 4; ++i) tot[i] = __builtin_fmaf(cur[i], sv, tot[i]);
     };
@@ -357,10 +391,20 @@ __global__ __launch_bounds__(256) void fp8b_mfma_gemv_kernel(const uint16_t* __r
 }
 
 constexpr size_t LDS_MAX = 160 * 1024;
+constexpr size_t MFMA_LDS_MAX = 120 * 1024;       // activations of the matrix-unit kernel (beside its 4 KB of sums)
 
 template <int FMT>
 int launch_qgemv(const void* x, const void* w, const void* sc, float* y, int m, int n, int k, int xs, int rpg, int bs, hipStream_t st)
 {
+    if (m >= 3 && k % 512 == 0 && n % 16 == 0 && rpg == 0 && (FMT != 2 || bs == 128)) {     // three or more rows: the matrix unit
+        const size_t smm = (size_t)m * (k + MG_PAD) * 2;
+        if (smm <= MFMA_LDS_MAX) {
+            static bool attr = hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess;
+            if (!attr) return 3;
+            q_mfma_gemv_kernel<FMT><<<n / 16, 256, smm, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
+            return launch_status();
+        }
+    }
     const size_t sm = (size_t)m * k * 2;
     if (sm > LDS_MAX) return 2;
     const dim3 b(64 * GEMV_WAVES);
@@ -443,13 +487,6 @@ SPARK_API int ds41_fp8_gemv(const void* x, const void* w, const void* ws, float*
 SPARK_API int spark_fp8_block128_gemv(const void* x, const void* w, const float* scales, float* y, int m, int n, int k, hipStream_t st)
 {
     if (m < 1 || m > 8 || n < 1 || k < 16 || k % 16 != 0) return 1;
-    if (m >= 3 && k % 512 == 0 && n % 16 == 0) {          // three or more rows: the matrix unit
-        const size_t sm = (size_t)m * (k + MG_PAD) * 2;
-        if (sm <= 64 * 1024) {
-            fp8b_mfma_gemv_kernel<<<n / 16, 256, sm, st>>>((const uint16_t*)x, (const uint8_t*)w, scales, y, m, n, k);
-            return launch_status();
-        }
-    }
     return launch_qgemv<2>(x, w, scales, y, m, n, k, k, 0, 128, st);
 }
 // reference ds41.cu:251-258: W bf16 [n, k]

@@ -164,6 +164,30 @@ def test_fp8_gemvs(ops, oracle, m):
     assert rel_l2(y, ref) < 1e-5
 
 
+@pytest.mark.parametrize("m,n,k", [(3, 208, 1536), (5, 64, 512), (8, 128, 4096), (4, 7168, 4096)])
+def test_matrix_unit_gemvs(ops, oracle, m, n, k):
+    # three or more rows of an eligible shape (k % 512 == 0, n % 16 == 0) run on the matrix unit in all three formats; the E8M0
+    # scales span 50 binades inside a K block (they are applied relative to the block's largest)
+    g = synth.rng(160 + m)
+    x = synth.randn_bf16(g, (m, k))
+    w4, s4 = synth.mxfp4_matrix(g, n, k, 119)
+    s4 = g.integers(80, 131, s4.shape, dtype=np.uint8)
+    y = host(ops.mxfp4_gemv(dev_bf16(x), dev(w4), dev(s4)))
+    ref = oracle.mxfp4_gemv(x, w4, s4)
+    assert np.abs(y - ref).max() / np.abs(ref).max() < 1e-5 and rel_l2(y, ref) < 1e-5
+    w8, sb = synth.fp8_block_matrix(g, n, k)
+    y = host(ops.fp8_block128_gemv(dev_bf16(x), dev(w8), dev(sb)))
+    ref = oracle.fp8_block_gemv(x, w8, sb)
+    assert np.abs(y - ref).max() / np.abs(ref).max() < 1e-5 and rel_l2(y, ref) < 1e-5
+    s8 = g.integers(80, 131, ((n + 31) // 32, k // 32), dtype=np.uint8)
+    y = host(ops.fp8_gemv(dev_bf16(x), dev(w8), dev(s8)))
+    ref = oracle.fp8_e8m0_gemv(x, w8, s8)
+    assert np.abs(y - ref).max() / np.abs(ref).max() < 1e-5 and rel_l2(y, ref) < 1e-5
+    if m > 3:                                                          # a row's value does not depend on the other rows
+        y3 = host(ops.fp8_gemv(dev_bf16(x[:3]), dev(w8), dev(s8)))
+        assert np.array_equal(y3, y[:3])
+
+
 def test_fp8_gemv_bx_up_to_16_rows_and_groups(ops, oracle):
     g = synth.rng(150)
     n, k, m = 256, 512, 13
