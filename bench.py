@@ -165,6 +165,7 @@ class Mxfp4Layer:
     H, I, E, TOPK, NS, LAYERS = 4096, 2048, 384, 6, 1, 61
     DTYPE = "fp4 x fp8 (E2M1 weights x E4M3 activations, E8M0 block scales, block-scaled MFMA, fp32 accumulate)"
     SET = "5.1 GB expert set"
+    TAG = "C3 deepseek-style"
 
     def __init__(self, torch, ops, R, inst, seed=1):
         self.torch, self.ops, self.R, self.inst = torch, ops, R, inst
@@ -187,7 +188,7 @@ class Mxfp4Layer:
         self.rw = torch.empty(inst, R, self.TOPK, dtype=torch.float32, device=dev)
         self.y = torch.empty(inst, R, H, dtype=torch.float32, device=dev)
         self.ws = ops.mxfp4_moe_ws_alloc(R, self.ex, self.TOPK)
-        self.name = f"C3 deepseek-style MXFP4 MoE layer (H {H}, I {I}, {self.E} experts top-{self.TOPK} + {self.NS} shared), batch {R}"
+        self.name = f"{self.TAG} MXFP4 MoE layer (H {H}, I {I}, {self.E} experts top-{self.TOPK} + {self.NS} shared), batch {R}"
 
     def step(self, i):
         ops, L = self.ops, self.ops._lib()
@@ -213,6 +214,7 @@ class Mxfp4LayerWide(Mxfp4Layer):
     ten 512-wide K groups for the eight waves of a gate/up block."""
     H = 5120
     SET = "6.4 GB expert set"
+    TAG = "reference-sized ds41"
 
 
 class Mxfp4Prefill(Mxfp4Layer):
