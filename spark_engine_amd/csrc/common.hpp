@@ -68,10 +68,23 @@ __device__ __forceinline__ uint32_t aq_scale(float amax)
     const uint32_t bits = __float_as_uint(amax * (1.0f / 448.0f));
     return ((bits >> 23) & 0xffu) + ((bits & 0x7fffffu) != 0u ? 1u : 0u);
 }
+// 1 / 2^(e - 127) as binary32: multiplying by it is the division by the scale, bit for bit (a power of two; 2^-127 is a
+// denormal, the reciprocal of the scale byte 255 - infinity - is 0)
+__device__ __forceinline__ float aq_inv(uint32_t e) { return __uint_as_float(e < 254u ? (254u - e) << 23 : (e == 254u ? 0x00400000u : 0u)); }
+__device__ __forceinline__ float aq_clamp(float v, float inv) { return fminf(fmaxf(v * inv, -448.f), 448.f); }
+// The encode is the hardware's (v_cvt_pk_fp8_f32: OCP E4M3, round to nearest even, denormal codes included; it turns what lies
+// beyond the format into NaN, which the clamp in front excludes): the same bytes as f32_to_e4m3 above, which every binary16
+// input of act_quant checks.
 __device__ __forceinline__ uint32_t aq_byte(float v, uint32_t e)
 {
-    const float s = __uint_as_float(e << 23);
-    return f32_to_e4m3(fminf(fmaxf(v / s, -448.f), 448.f));
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(aq_clamp(v, aq_inv(e)), 0.f, 0, false) & 0xffu;
+}
+// four values under one scale -> four code bytes, v0 in the low byte
+__device__ __forceinline__ uint32_t aq_word4(float v0, float v1, float v2, float v3, uint32_t e)
+{
+    const float inv = aq_inv(e);
+    const int lo = __builtin_amdgcn_cvt_pk_fp8_f32(aq_clamp(v0, inv), aq_clamp(v1, inv), 0, false);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(aq_clamp(v2, inv), aq_clamp(v3, inv), lo, true);
 }
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
 

@@ -124,10 +124,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t* __restri
     a = fmaxf(a, __shfl_xor(a, 2, 64));
     const uint32_t e = aq_scale(a);
     if (BYTES) {
-        uint32_t lo = 0, hi = 0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { lo |= aq_byte(v[i], e) << (8 * i); hi |= aq_byte(v[4 + i], e) << (8 * i); }
-        *(uint2*)(q + t * 8) = make_uint2(lo, hi);
+        *(uint2*)(q + t * 8) = make_uint2(aq_word4(v[0], v[1], v[2], v[3], e), aq_word4(v[4], v[5], v[6], v[7], e));
         if ((t & 3) == 0) s[b] = (uint8_t)e;
     } else {
         uint32_t o[4];

@@ -172,9 +172,7 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void fp8q_gemv_kernel(const uint16
             am = fmaxf(am, lane_xor<1>(am, lane));
             am = fmaxf(am, lane_xor<2>(am, lane));
             e = aq_scale(am);
-            code[0] = code[1] = 0;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) { code[0] |= aq_byte(v[j], e) << (8 * j); code[1] |= aq_byte(v[4 + j], e) << (8 * j); }
+            code[0] = aq_word4(v[0], v[1], v[2], v[3], e); code[1] = aq_word4(v[4], v[5], v[6], v[7], e);
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) xl[(size_t)r * k + c + j] = f32_to_bf16(e4m3_to_f32((code[j >> 2] >> (8 * (j & 3))) & 0xffu));

@@ -619,10 +619,7 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
         const uint32_t e = aq_scale(fmaxf(amx[wave][rt][c], amx[wave ^ 1][rt][c]));
-        uint32_t word = 0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) word |= aq_byte(yv[rt][i], e) << (8 * i);
-        *(uint32_t*)&hbuf[rt * 16 + c][16 * wave + 4 * rg] = word;
+        *(uint32_t*)&hbuf[rt * 16 + c][16 * wave + 4 * rg] = aq_word4(yv[rt][0], yv[rt][1], yv[rt][2], yv[rt][3], e);
         if (rg == 0 && (wave & 1) == 0) hes[rt * 16 + c][wave >> 1] = (unsigned char)e;
     }
     __syncthreads();

@@ -155,10 +155,7 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
                         am = fmaxf(am, lane_xor<1>(am, lane));
                         am = fmaxf(am, lane_xor<2>(am, lane));
                         const uint32_t e = aq_scale(am);
-                        uint32_t lo = 0, hi = 0;
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) { lo |= aq_byte(v[i], e) << (8 * i); hi |= aq_byte(v[4 + i], e) << (8 * i); }
-                        *(uint2*)(xql + (size_t)r * H + k) = make_uint2(lo, hi);
+                        *(uint2*)(xql + (size_t)r * H + k) = make_uint2(aq_word4(v[0], v[1], v[2], v[3], e), aq_word4(v[4], v[5], v[6], v[7], e));
                         if ((lane & 3) == 0) xsl[(size_t)r * (H >> 5) + (k >> 5)] = (unsigned char)e;
                     }
                 }
