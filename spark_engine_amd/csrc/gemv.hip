@@ -388,6 +388,104 @@ __global__ __launch_bounds__(256) void q_mfma_gemv_kernel(const uint16_t* __rest
     }
 }
 
+// The same product on the matrix unit: v_mfma_scale_f32_16x16x128_f8f6f4 multiplies E4M3 by E4M3 with an E8M0 scale per 32 k on
+// either side, which is this format exactly (the products and scales are exact, the sums binary32).  Workgroup = 16 weight rows,
+// wave = a quarter of K; a lane's A operand of a 128-wide step is two 16-byte loads of its row (k = 16 g + e and 64 + 16 g + e),
+// four steps in flight; the activation codes and scales (given, or quantised here by the rule of act_quant) sit in LDS with
+// row strides that spread the 16 rows over the banks.  Up to 16 activation rows per launch: the columns of the tile.  The four
+// K quarters are summed through LDS in wave order.  A row's value does not depend on the rows beside it.
+constexpr int FQ_CPAD = 16, FQ_SPAD = 4;
+template <bool QUANT>
+__global__ __launch_bounds__(256) void fp8q_mfma_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ aq, const uint8_t* __restrict__ as_,
+                                                        const uint8_t* __restrict__ w, const uint8_t* __restrict__ ws, void* __restrict__ y, int ob16, int m, int n,
+                                                        int k)
+{
+    extern __shared__ __align__(16) unsigned char fq_lds[];
+    __shared__ float red[4][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
+    const int cld = k + FQ_CPAD, nb32 = k >> 5, sld = nb32 + FQ_SPAD;
+    unsigned char* xc = fq_lds;                           // [m][k + pad] codes
+    unsigned char* xs = fq_lds + (size_t)m * cld;         // [m][k / 32 + pad] scale bytes
+    const int n0 = blockIdx.x * 16;
+    const int ks = k / 4, kb0 = wave * ks, nstep = ks / 128;
+    const uint8_t* wp = w + (int64_t)(n0 + c) * k + kb0 + 16 * g;
+    const uint8_t* sp = ws + (int64_t)(n0 >> 5) * nb32 + kb0 / 32;        // the tile's 16 rows share a 32-row scale group
+    uint4 a[4][2], sq;
+    auto fetch = [&](auto uc, int st) {
+        constexpr int u = decltype(uc)::value;
+        a[u][0] = ld_stream16(wp + st * 128); a[u][1] = ld_stream16(wp + st * 128 + 64);
+    };
+    fetch(std::integral_constant<int, 0>{}, 0);
+    fetch(std::integral_constant<int, 1>{}, min(1, nstep - 1));
+    fetch(std::integral_constant<int, 2>{}, min(2, nstep - 1));
+    fetch(std::integral_constant<int, 3>{}, min(3, nstep - 1));
+    sq = *(const uint4*)sp;                                // the scale bytes of four steps (16 blocks), the same for every lane
+    if (QUANT) {
+        for (int i = threadIdx.x; i < m * nb32 * 4; i += 256) {            // 4 threads per 32-block, 8 elements each
+            const int r = i / (nb32 * 4), q = i % (nb32 * 4), b = q >> 2, col = b * 32 + (q & 3) * 8;
+            const uint4 raw = *(const uint4*)(x + (int64_t)r * k + col);
+            const uint32_t rw4[4] = {raw.x, raw.y, raw.z, raw.w};
+            float v[8], am = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[2 * j] = __uint_as_float(rw4[j] << 16); v[2 * j + 1] = __uint_as_float(rw4[j] & 0xffff0000u);
+                am = fmaxf(am, fmaxf(fabsf(v[2 * j]), fabsf(v[2 * j + 1])));
+            }
+            am = fmaxf(am, lane_xor<1>(am, lane));
+            am = fmaxf(am, lane_xor<2>(am, lane));
+            const uint32_t e = aq_scale(am);
+            *(uint2*)(xc + (size_t)r * cld + col) = make_uint2(aq_word4(v[0], v[1], v[2], v[3], e), aq_word4(v[4], v[5], v[6], v[7], e));
+            if ((q & 3) == 0) xs[r * sld + b] = (unsigned char)e;
+        }
+    } else {
+        const int n16 = k / 16;
+        for (int i = threadIdx.x; i < m * n16; i += 256) {
+            const int r = i / n16, col = (i % n16) * 16;
+            *(uint4*)(xc + (size_t)r * cld + col) = *(const uint4*)(aq + (int64_t)r * k + col);
+        }
+        for (int i = threadIdx.x; i < m * (nb32 / 4); i += 256) {
+            const int r = i / (nb32 / 4), col = (i % (nb32 / 4)) * 4;
+            *(uint32_t*)(xs + r * sld + col) = *(const uint32_t*)(as_ + (int64_t)r * nb32 + col);
+        }
+    }
+    __syncthreads();
+    const int br = min(c, m - 1);
+    const unsigned char* bc = xc + (size_t)br * cld + kb0 + 16 * g;
+    const unsigned char* bs = xs + br * sld + kb0 / 32;
+    v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+    auto step = [&](auto uc, int st) {
+        constexpr int u = decltype(uc)::value;
+        const uint4 lo = *(const uint4*)(bc + st * 128), hi = *(const uint4*)(bc + st * 128 + 64);
+        const v8i b8 = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+        const v8i a8 = v8i{(int)a[u][0].x, (int)a[u][0].y, (int)a[u][0].z, (int)a[u][0].w, (int)a[u][1].x, (int)a[u][1].y, (int)a[u][1].z, (int)a[u][1].w};
+        const uint32_t sdw = u == 0 ? sq.x : u == 1 ? sq.y : u == 2 ? sq.z : sq.w;
+        const uint32_t sa = (sdw >> (8 * g)) & 0xffu;
+        const uint32_t sb = (*(const uint32_t*)(bs + st * 4) >> (8 * g)) & 0xffu;
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc, 0 /*A: E4M3*/, 0 /*B: E4M3*/, 0, (int)sa, 0, (int)sb);
+        fetch(uc, min(st + 4, nstep - 1));                // four steps ahead, into the registers just used
+    };
+    for (int st = 0; st < nstep; st += 4) {
+        const uint4 sqn = *(const uint4*)(sp + min(st + 4, nstep - 1) / 4 * 16);
+        step(std::integral_constant<int, 0>{}, st);
+        if (st + 1 < nstep) step(std::integral_constant<int, 1>{}, st + 1);
+        if (st + 2 < nstep) step(std::integral_constant<int, 2>{}, st + 2);
+        if (st + 3 < nstep) step(std::integral_constant<int, 3>{}, st + 3);
+        sq = sqn;
+    }
+    // D: lane = activation row c, output rows n0 + 4 g + i
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
+    __syncthreads();
+    if (wave == 0 && c < m) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float v = ((red[0][lane][i] + red[1][lane][i]) + red[2][lane][i]) + red[3][lane][i];
+            const int64_t o = (int64_t)c * n + n0 + 4 * g + i;
+            if (ob16) ((uint16_t*)y)[o] = f32_to_bf16(v); else ((float*)y)[o] = v;
+        }
+    }
+}
+
 constexpr size_t LDS_MAX = 160 * 1024;
 constexpr size_t MFMA_LDS_MAX = 120 * 1024;       // activations of the matrix-unit kernel (beside its 4 KB of sums)
 
@@ -445,6 +543,24 @@ SPARK_API int ds41_fp8_gemv_mx_q(const void* x, const void* aq, const void* as_,
                                  hipStream_t st)
 {
     if (m < 1 || m > 32 || k % 64 || n % 8 || (!x && !aq) || (aq && !as_)) return 1;
+    if (k % 2048 == 0 && n % 16 == 0) {                    // the matrix unit: whole steps of 128 per K quarter, four at a time; whole 16-row tiles (each inside one 32-row scale group)
+        const auto need = [&](int rows) { return (size_t)rows * (k + FQ_CPAD) + (size_t)rows * (k / 32 + FQ_SPAD); };
+        const int per = need(16) <= 80 * 1024 ? 16 : need(8) <= 80 * 1024 ? 8 : 0;      // two workgroups per CU
+        if (per) {
+            static bool attr = hipFuncSetAttribute((const void*)fp8q_mfma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) == hipSuccess &&
+                               hipFuncSetAttribute((const void*)fp8q_mfma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) == hipSuccess;
+            if (!attr) return 3;
+            for (int r0 = 0; r0 < m; r0 += per) {
+                const int mm = m - r0 < per ? m - r0 : per;
+                void* yr = ob16 ? (void*)((uint16_t*)y + (int64_t)r0 * n) : (void*)((float*)y + (int64_t)r0 * n);
+                if (aq) fp8q_mfma_kernel<false><<<n / 16, 256, need(mm), st>>>(nullptr, (const uint8_t*)aq + (int64_t)r0 * k, (const uint8_t*)as_ + (int64_t)r0 * (k / 32),
+                                                                                (const uint8_t*)w, (const uint8_t*)ws, yr, ob16, mm, n, k);
+                else fp8q_mfma_kernel<true><<<n / 16, 256, need(mm), st>>>((const uint16_t*)x + (int64_t)r0 * k, nullptr, nullptr, (const uint8_t*)w, (const uint8_t*)ws,
+                                                                           yr, ob16, mm, n, k);
+            }
+            return launch_status();
+        }
+    }
     const dim3 g((n + GEMV_WAVES * RPW - 1) / (GEMV_WAVES * RPW)), b(64 * GEMV_WAVES);
     for (int r0 = 0; r0 < m; r0 += 8) {
         const int mm = m - r0 < 8 ? m - r0 : 8;

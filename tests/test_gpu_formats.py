@@ -208,12 +208,13 @@ def test_fp8_gemv_bx_up_to_16_rows_and_groups(ops, oracle):
         assert rel_l2(yg[:, 64 * j:64 * j + 64], refj) < 1e-5
 
 
-def test_fp8_gemv_with_quantised_activations(ops, oracle):
-    # FP8 weights x act-quantised activations: every product is exact, the reference is the same sum in float64
+@pytest.mark.parametrize("n,k,m", [(256, 1024, 11), (208, 2048, 21), (64, 4096, 3), (7168, 4096, 16)])
+def test_fp8_gemv_with_quantised_activations(ops, oracle, n, k, m):
+    # FP8 weights x act-quantised activations: every product is exact, the reference is the same sum in float64.  k a multiple of
+    # 2048 with n a multiple of 16 runs on the matrix unit (16 rows per launch), the first shape on the dot-product kernel
     g = synth.rng(151)
-    n, k, m = 256, 1024, 11
     w8, _ = synth.fp8_block_matrix(g, n, k)
-    s8 = g.integers(110, 128, (n // 32, k // 32), dtype=np.uint8)
+    s8 = g.integers(110, 128, ((n + 31) // 32, k // 32), dtype=np.uint8)
     x = synth.randn_bf16(g, (m, k))
     q, s = oracle.act_quant_fp8(x)
     W = oracle.fp8_e8m0_dequant(w8, s8).astype(np.float64)
@@ -226,8 +227,8 @@ def test_fp8_gemv_with_quantised_activations(ops, oracle):
     assert np.array_equal(y, y2)                                         # quantised inside = quantised by the caller
     yb = host(ops.fp8_gemv_mx(dev_bf16(x), dev(w8), dev(s8), bf16_out=True))
     assert np.array_equal(yb, synth.bf16_bits(y))
-    y1 = host(ops.fp8_gemv_mx(dev_bf16(x[3:4]), dev(w8), dev(s8)))
-    assert np.array_equal(y1[0], y[3])                                   # a row's value does not depend on the row count
+    y1 = host(ops.fp8_gemv_mx(dev_bf16(x[2:3]), dev(w8), dev(s8)))
+    assert np.array_equal(y1[0], y[2])                                   # a row's value does not depend on the row count
 
 
 def test_gemv_rejects_bad_shapes(ops):
