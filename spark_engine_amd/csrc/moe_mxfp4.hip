@@ -439,11 +439,15 @@ constexpr int GT_FEAT = 128;           // output features / columns of a block
 //   PACK8 / MX8 (reference engine-rs/src/ds41/kern.rs moe_pack / moe_pack_mx): tiles of 8 rows, [K / 128][8][64 bytes] codes and
 //   [K / 128][8][4] scales.  MX8 keeps a row's 64 bytes as 4 x 4 dwords [q][b] and the lane of K block g needs column b = g: the
 //   four lanes of a row (16 apart) load one q-row each and transpose with two rounds of row swaps.  The scale dword is gathered
-//   the same way: lane (row, g) loads the four block scales of step g and the four lanes transpose 4 x 4 bytes.
+//   the same way: lane (row, g) loads the four block scales of step g and the four lanes transpose 4 x 4 bytes.  MX8S2: the
+//   codes of MX8 with the scales in the lossless 2-bit coding (a base byte per row + four 2-bit offsets per step, or raw words).
 template <int LAYOUT> struct ATile {
     const uint8_t* w;
-    const uint8_t* sc;
-    static constexpr int KGW = LAYOUT == L_T16 ? REC : 2048, STEPW = LAYOUT == L_T16 ? 1024 : 512, KGS = LAYOUT == L_T16 ? REC : 128;
+    const uint8_t* sc;                 // MX8S2: this lane's code byte of K group 0 (step g, row of the tile)
+    const uint8_t* raw;                // MX8S2: the tile's raw scale words when it has them (else null)
+    uint32_t base4;                    // MX8S2: the row's base scale in all four bytes
+    static constexpr bool MXT = LAYOUT == L_MX8 || LAYOUT == L_MX8S2;       // 4 x 4 dword order inside a row's 64 bytes
+    static constexpr int KGW = LAYOUT == L_T16 ? REC : 2048, STEPW = LAYOUT == L_T16 ? 1024 : 512, KGS = LAYOUT == L_T16 ? REC : LAYOUT == L_MX8S2 ? 32 : 128;
     __device__ __forceinline__ ATile(const WMat& m, int64_t row0, int lane)          // row0: first row of the tile in the stacked matrix
     {
         const int steps = m.K >> 7;
@@ -454,7 +458,15 @@ template <int LAYOUT> struct ATile {
             const int64_t row = row0 + (lane & 15), t8 = row >> 3;
             const int r8 = (int)(row & 7), g = lane >> 4;
             w = m.w + t8 * steps * 512 + r8 * 64 + g * 16;
-            sc = m.s + t8 * steps * 32 + g * 32 + r8 * 4;
+            if constexpr (LAYOUT == L_MX8S2) {
+                // the lossless 2-bit coding (reference engine-rs/shim/ds41_mx.cu:64-91): desc [T][16], codes [T][S][8], raw [n_raw][S][8][4]
+                const uint32_t* d = (const uint32_t*)(m.s + t8 * 16);
+                const uint8_t* code = m.s + m.tiles8 * 16;
+                const int ri = (int)d[2];
+                base4 = ((d[r8 >> 2] >> (8 * (r8 & 3))) & 0xffu) * 0x01010101u;
+                sc = code + (t8 * steps + g) * 8 + r8;
+                raw = ri >= 0 ? code + m.tiles8 * steps * 8 + ((int64_t)ri * steps + g) * 32 + r8 * 4 : nullptr;
+            } else sc = m.s + t8 * steps * 32 + g * 32 + r8 * 4;
         }
     }
     __device__ __forceinline__ v4i codes(int kg, int s) const
@@ -464,7 +476,7 @@ template <int LAYOUT> struct ATile {
     }
     __device__ __forceinline__ static v4i fix(const v4i& v)
     {
-        if constexpr (LAYOUT != L_MX8) return v;
+        if constexpr (!MXT) return v;
         else {
             const auto a02 = __builtin_amdgcn_permlane32_swap((uint32_t)v.x, (uint32_t)v.z, false, false);
             const auto a13 = __builtin_amdgcn_permlane32_swap((uint32_t)v.y, (uint32_t)v.w, false, false);
@@ -473,7 +485,18 @@ template <int LAYOUT> struct ATile {
             return v4i{(int)b01[0], (int)b01[1], (int)b23[0], (int)b23[1]};
         }
     }
-    __device__ __forceinline__ uint32_t scales_raw(int kg) const { return *(const uint32_t*)(sc + (int64_t)kg * KGS); }
+    __device__ __forceinline__ uint32_t scales_raw(int kg) const
+    {
+        if constexpr (LAYOUT == L_MX8S2) {
+            // both forms are requested whatever the tile has (no load behind a branch): a tile without raw words reads its code
+            // byte's word a second time
+            const uint8_t* cp = sc + (int64_t)kg * KGS;
+            const uint32_t cb = *cp;
+            const uint32_t rw = *(const uint32_t*)(raw ? raw + (int64_t)kg * 128 : (const uint8_t*)((uintptr_t)cp & ~(uintptr_t)3));
+            const uint32_t coded = base4 + ((cb & 3u) | ((cb & 0xcu) << 6) | ((cb & 0x30u) << 12) | ((cb & 0xc0u) << 18));
+            return raw ? rw : coded;
+        } else return *(const uint32_t*)(sc + (int64_t)kg * KGS);
+    }
     // what scales_raw() loaded -> byte s = the scale of this lane's K block in step s
     __device__ __forceinline__ static uint32_t scales_fix(uint32_t d, int lane)
     {
@@ -490,7 +513,7 @@ template <int LAYOUT> struct ATile {
         }
     }
 };
-constexpr bool gemm_layout(int layout) { return layout == L_T16 || layout == L_PACK8 || layout == L_MX8; }
+constexpr bool gemm_layout(int layout) { return layout == L_T16 || layout == L_PACK8 || layout == L_MX8 || layout == L_MX8S2; }
 
 // Visit order of the K groups of a gate / up product with more than eight of them: the decode kernels' wave s (of eight) walks K
 // groups s, s + 8 in one accumulator and the eight sums are added in wave order, so visit i is K group kg, `fresh` says that it

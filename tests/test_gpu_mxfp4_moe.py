@@ -225,3 +225,17 @@ def test_ds41_two_bit_coded_scales(ops, oracle):
         ops.moe_s2_set(False)
     assert np.array_equal(host(y_s2), host(y_raw))
     assert rel_l2(host(y_s2), ref) <= TOL
+    # more than 8 rows: the grouped GEMM decodes the same blobs (coded tiles and the raw one)
+    R2 = 40
+    x2 = synth.randn_bf16(g, (R2, H))
+    idx2 = np.stack([g.permutation(E)[:topk] for _ in range(R2)]).astype(np.int64)
+    rw2 = g.uniform(0.1, 1.0, (R2, topk)).astype(np.float32)
+    xq2, xs2 = ops.act_quant_fp8(dev_bf16(x2))
+    y2_raw, _ = ops.ds41_moe_mx(xq2, xs2, dev(idx2), dev(rw2), (packed[0], ps1, packed[1], ps3, packed[2], ps2), I)
+    ops.moe_s2_set(True)
+    try:
+        y2_s2, _ = ops.ds41_moe_mx(xq2, xs2, dev(idx2), dev(rw2), (packed[0], b1, packed[1], b3, packed[2], b2), I)
+    finally:
+        ops.moe_s2_set(False)
+    assert np.array_equal(host(y2_s2), host(y2_raw))
+    assert rel_l2(host(y2_s2), oracle.mxfp4_moe(x2, idx2, rw2, *ws)) <= TOL
