@@ -269,6 +269,111 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void bf16_gemv_kernel(const uint16
     }
 }
 
+// Up to four activation rows on matrices of whole 16-row tiles: workgroup = 16 weight rows, wave = one span of K (64 lanes x 16
+// bytes) of all 16 rows.  Every load instruction reads 1 KB of one row, all 16 are in flight at once, and a lane's activations
+// (the same k for its 16 rows) come straight from memory once: no LDS staging, no barrier before the first multiply.  Measured
+// against the rows-per-wave order above on 7168 x 4096 bytes, reads alone: 5.8 vs 6.8 us; the kernels at one row: 6.4 vs 8.5 us.
+// The 16 row sums of a wave are folded across lanes by halving (8 + 4 + 2 + 1 exchanges, then 2 more), the K spans are added
+// through LDS in wave order.
+template <int FMT, int M>
+__global__ __launch_bounds__(512) void rowtile_gemv_kernel(const uint16_t* __restrict__ x, int64_t xs, const uint8_t* __restrict__ w, const void* __restrict__ scv,
+                                                           float* __restrict__ y, int m, int n, int k, int bs)
+{
+    __shared__ float red[8][M][16];
+    constexpr int EPP = FMT == 0 ? 32 : 16;               // elements per 16-byte piece
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int n0 = blockIdx.x * 16, e0 = wave * 64 * EPP + lane * EPP;     // this lane's first k
+    const int64_t rb = FMT == 0 ? k / 2 : k;
+    const uint8_t* wp = w + (int64_t)n0 * rb + (FMT == 0 ? e0 / 2 : e0);
+    uint4 p[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) p[i] = ld_stream16(wp + i * rb);
+    // scales: one per lane for the block formats (the tile's rows share a scale block), one per row for MXFP4
+    float sc1 = 1.0f;
+    uint32_t sb[FMT == 0 ? 16 : 1];
+    if constexpr (FMT == 2) sc1 = ((const float*)scv)[(int64_t)(n0 / bs) * ((k + bs - 1) / bs) + e0 / bs];
+    else if constexpr (FMT == 1) sc1 = e8m0_to_f32(((const uint8_t*)scv)[(int64_t)(n0 >> 5) * (k >> 5) + (e0 >> 5)]);
+    else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sb[i] = ((const uint8_t*)scv)[(int64_t)(n0 + i) * (k >> 5) + (e0 >> 5)];
+    }
+    uint4 xv[M][EPP / 8];
+#pragma unroll
+    for (int r = 0; r < M; ++r)
+#pragma unroll
+        for (int j = 0; j < EPP / 8; ++j) xv[r][j] = *(const uint4*)(x + (int64_t)(r < m ? r : m - 1) * xs + e0 + 8 * j);
+    float acc[M][16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t pw[4] = {p[i].x, p[i].y, p[i].z, p[i].w};
+        bf2 wv[EPP / 2];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (FMT == 0) {
+                wv[4 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 0);
+                wv[4 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 1);
+                wv[4 * j + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 2);
+                wv[4 * j + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], 1.0f, 3);
+            } else {
+                wv[2 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, false);
+                wv[2 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(pw[j], 1.0f, true);
+            }
+        }
+        const float sv = FMT == 0 ? e8m0_to_f32(sb[FMT == 0 ? i : 0]) : sc1;
+#pragma unroll
+        for (int r = 0; r < M; ++r) {
+            float t = 0.f;
+#pragma unroll
+            for (int j = 0; j < EPP / 8; ++j) {
+                t = __builtin_amdgcn_fdot2_f32_bf16(wv[4 * j + 0], as_bf2(xv[r][j].x), t, false);
+                t = __builtin_amdgcn_fdot2_f32_bf16(wv[4 * j + 1], as_bf2(xv[r][j].y), t, false);
+                t = __builtin_amdgcn_fdot2_f32_bf16(wv[4 * j + 2], as_bf2(xv[r][j].z), t, false);
+                t = __builtin_amdgcn_fdot2_f32_bf16(wv[4 * j + 3], as_bf2(xv[r][j].w), t, false);
+            }
+            acc[r][i] = t * sv;
+        }
+    }
+    // fold: after the step with partner distance d a lane keeps the rows whose bit d matches its own lane bit
+#pragma unroll
+    for (int r = 0; r < M; ++r) {
+        float v8[8], v4[4], v2[2], v1;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const bool up = (lane & 1) != 0;
+            const float keep = up ? acc[r][2 * i + 1] : acc[r][2 * i], give = up ? acc[r][2 * i] : acc[r][2 * i + 1];
+            v8[i] = keep + lane_xor<1>(give, lane);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool up = (lane & 2) != 0;
+            const float keep = up ? v8[2 * i + 1] : v8[2 * i], give = up ? v8[2 * i] : v8[2 * i + 1];
+            v4[i] = keep + lane_xor<2>(give, lane);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const bool up = (lane & 4) != 0;
+            const float keep = up ? v4[2 * i + 1] : v4[2 * i], give = up ? v4[2 * i] : v4[2 * i + 1];
+            v2[i] = keep + lane_xor<4>(give, lane);
+        }
+        {
+            const bool up = (lane & 8) != 0;
+            const float keep = up ? v2[1] : v2[0], give = up ? v2[0] : v2[1];
+            v1 = keep + lane_xor<8>(give, lane);
+        }
+        v1 += lane_xor<16>(v1, lane);
+        v1 += lane_xor<32>(v1, lane);
+        // every lane now holds the wave's sum of row (lane & 15)
+        if (lane < 16) red[wave][r][lane] = v1;
+    }
+    __syncthreads();
+    if (threadIdx.x < 16 * M) {
+        const int r = threadIdx.x >> 4, i = threadIdx.x & 15;
+        float v = red[0][r][i];
+        for (int u = 1; u < nw; ++u) v += red[u][r][i];
+        if (r < m) y[(int64_t)r * n + n0 + i] = v;
+    }
+}
+
 // Three or more activation rows: the matrix unit does the multiplies (with one or two rows the dot-product kernel above is as
 // fast and keeps its summation order).  Wave = 16 output rows x a quarter of K: a lane's piece of a 128-wide K block holds 32
 // neighbouring k of one row (two 16-byte loads of E4M3, one of E2M1), converted to bf16 pairs (exact) and fed as the A operand of
@@ -494,6 +599,18 @@ constexpr size_t MFMA_LDS_MAX = 120 * 1024;       // activations of the matrix-u
 template <int FMT>
 int launch_qgemv(const void* x, const void* w, const void* sc, float* y, int m, int n, int k, int xs, int rpg, int bs, hipStream_t st)
 {
+    {
+        // the row-tile kernel: up to four rows of the FP8 formats, up to two of MXFP4 (whose spans are 2048 wide: four of them or more)
+        constexpr int SPAN = 64 * (FMT == 0 ? 32 : 16);
+        const int nw = k / SPAN;
+        if (m <= (FMT == 0 ? 2 : 4) && rpg == 0 && n % 16 == 0 && k % SPAN == 0 && nw >= (FMT == 0 ? 4 : 2) && nw <= 8 && xs % 8 == 0 &&
+            (FMT != 2 || (bs >= 16 && bs % 16 == 0))) {
+            if (m == 1) rowtile_gemv_kernel<FMT, 1><<<n / 16, 64 * nw, 0, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k, bs);
+            else if (m == 2) rowtile_gemv_kernel<FMT, 2><<<n / 16, 64 * nw, 0, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k, bs);
+            else rowtile_gemv_kernel<FMT, 4><<<n / 16, 64 * nw, 0, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k, bs);
+            return launch_status();
+        }
+    }
     if (m >= 3 && k % 512 == 0 && n % 16 == 0 && rpg == 0 && (FMT != 2 || bs == 128)) {     // three or more rows: the matrix unit
         const size_t smm = (size_t)m * (k + MG_PAD) * 2;
         if (smm <= MFMA_LDS_MAX) {
