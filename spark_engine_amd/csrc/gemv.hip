@@ -497,11 +497,12 @@ __global__ __launch_bounds__(64 * KW) void q_mfma_gemv_kernel(const uint16_t* __
 
 // The same product on the matrix unit: v_mfma_scale_f32_16x16x128_f8f6f4 multiplies E4M3 by E4M3 with an E8M0 scale per 32 k on
 // either side, which is this format exactly (the products and scales are exact, the sums binary32).  Workgroup = 16 weight rows,
-// wave = a quarter of K; a lane's A operand of a 128-wide step is two 16-byte loads of its row (k = 16 g + e and 64 + 16 g + e),
-// four steps in flight; the activation codes and scales (given, or quantised here by the rule of act_quant) sit in LDS with
+// wave = a quarter of K; a lane's A operand of a 128-wide step is 16 bytes at k = 16 g and 16 at 64 + 16 g of its row, two
+// chunks of 256 k in flight; the activation codes and scales (given, or quantised here by the rule of act_quant) sit in LDS with
 // row strides that spread the 16 rows over the banks.  Up to 16 activation rows per launch: the columns of the tile.  The four
 // K quarters are summed through LDS in wave order.  A row's value does not depend on the rows beside it.
 constexpr int FQ_CPAD = 16, FQ_SPAD = 4;
+constexpr int FQ_TS = 256 + 16;        // row stride of a wave's transpose tile: 16-byte reads down its 16 rows hit distinct banks
 template <bool QUANT>
 __global__ __launch_bounds__(256) void fp8q_mfma_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ aq, const uint8_t* __restrict__ as_,
                                                         const uint8_t* __restrict__ w, const uint8_t* __restrict__ ws, void* __restrict__ y, int ob16, int m, int n,
@@ -515,17 +516,21 @@ __global__ __launch_bounds__(256) void fp8q_mfma_kernel(const uint16_t* __restri
     unsigned char* xs = fq_lds + (size_t)m * cld;         // [m][k / 32 + pad] scale bytes
     const int n0 = blockIdx.x * 16;
     const int ks = k / 4, kb0 = wave * ks, nstep = ks / 128;
-    const uint8_t* wp = w + (int64_t)(n0 + c) * k + kb0 + 16 * g;
+    // Weight loads: one instruction reads 256 bytes of each of four rows (lane l: row 4 i + l / 16, bytes 16 (l % 16) of the
+    // chunk), whole lines side by side - 64-byte pieces of 16 rows per instruction, the operand's own order, read a third slower.
+    // The chunk goes through a wave-private LDS tile into the operand order (lane = row c, K block g).
+    const int lr = lane >> 4, lc = (lane & 15) * 16, nchunk = nstep / 2;
+    const uint8_t* wp = w + (int64_t)(n0 + lr) * k + kb0 + lc;
+    unsigned char* tw = fq_lds + (((size_t)m * cld + (size_t)m * sld + 15) & ~(size_t)15) + (size_t)wave * (16 * FQ_TS);
     const uint8_t* sp = ws + (int64_t)(n0 >> 5) * nb32 + kb0 / 32;        // the tile's 16 rows share a 32-row scale group
-    uint4 a[4][2], sq;
-    auto fetch = [&](auto uc, int st) {
+    uint4 a[2][4], sq;
+    auto fetch = [&](auto uc, int ch) {
         constexpr int u = decltype(uc)::value;
-        a[u][0] = ld_stream16(wp + st * 128); a[u][1] = ld_stream16(wp + st * 128 + 64);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[u][i] = ld_stream16(wp + (int64_t)(4 * i) * k + ch * 256);
     };
     fetch(std::integral_constant<int, 0>{}, 0);
-    fetch(std::integral_constant<int, 1>{}, min(1, nstep - 1));
-    fetch(std::integral_constant<int, 2>{}, min(2, nstep - 1));
-    fetch(std::integral_constant<int, 3>{}, min(3, nstep - 1));
+    fetch(std::integral_constant<int, 1>{}, min(1, nchunk - 1));
     sq = *(const uint4*)sp;                                // the scale bytes of four steps (16 blocks), the same for every lane
     if (QUANT) {
         for (int i = threadIdx.x; i < m * nb32 * 4; i += 256) {            // 4 threads per 32-block, 8 elements each
@@ -560,23 +565,34 @@ __global__ __launch_bounds__(256) void fp8q_mfma_kernel(const uint16_t* __restri
     const unsigned char* bc = xc + (size_t)br * cld + kb0 + 16 * g;
     const unsigned char* bs = xs + br * sld + kb0 / 32;
     v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
-    auto step = [&](auto uc, int st) {
+    auto chunk = [&](auto uc, int ch) {                    // two steps of 128
         constexpr int u = decltype(uc)::value;
-        const uint4 lo = *(const uint4*)(bc + st * 128), hi = *(const uint4*)(bc + st * 128 + 64);
-        const v8i b8 = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-        const v8i a8 = v8i{(int)a[u][0].x, (int)a[u][0].y, (int)a[u][0].z, (int)a[u][0].w, (int)a[u][1].x, (int)a[u][1].y, (int)a[u][1].z, (int)a[u][1].w};
-        const uint32_t sdw = u == 0 ? sq.x : u == 1 ? sq.y : u == 2 ? sq.z : sq.w;
-        const uint32_t sa = (sdw >> (8 * g)) & 0xffu;
-        const uint32_t sb = (*(const uint32_t*)(bs + st * 4) >> (8 * g)) & 0xffu;
-        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc, 0 /*A: E4M3*/, 0 /*B: E4M3*/, 0, (int)sa, 0, (int)sb);
-        fetch(uc, min(st + 4, nstep - 1));                // four steps ahead, into the registers just used
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *(uint4*)(tw + (4 * i + lr) * FQ_TS + lc) = a[u][i];
+        __builtin_amdgcn_wave_barrier();                   // the tile belongs to this wave: its LDS operations execute in order
+        asm volatile("" ::: "memory");
+        uint4 al[2][2];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) { al[s2][0] = *(const uint4*)(tw + c * FQ_TS + s2 * 128 + 16 * g); al[s2][1] = *(const uint4*)(tw + c * FQ_TS + s2 * 128 + 64 + 16 * g); }
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+        fetch(uc, min(ch + 2, nchunk - 1));                // two chunks ahead, into the registers just used
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const int st = ch * 2 + s2;
+            const uint4 lo = *(const uint4*)(bc + st * 128), hi = *(const uint4*)(bc + st * 128 + 64);
+            const v8i b8 = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+            const v8i a8 = v8i{(int)al[s2][0].x, (int)al[s2][0].y, (int)al[s2][0].z, (int)al[s2][0].w, (int)al[s2][1].x, (int)al[s2][1].y, (int)al[s2][1].z, (int)al[s2][1].w};
+            const uint32_t sdw = u == 0 ? (s2 ? sq.y : sq.x) : (s2 ? sq.w : sq.z);
+            const uint32_t sa = (sdw >> (8 * g)) & 0xffu;
+            const uint32_t sb = (*(const uint32_t*)(bs + st * 4) >> (8 * g)) & 0xffu;
+            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc, 0 /*A: E4M3*/, 0 /*B: E4M3*/, 0, (int)sa, 0, (int)sb);
+        }
     };
-    for (int st = 0; st < nstep; st += 4) {
-        const uint4 sqn = *(const uint4*)(sp + min(st + 4, nstep - 1) / 4 * 16);
-        step(std::integral_constant<int, 0>{}, st);
-        if (st + 1 < nstep) step(std::integral_constant<int, 1>{}, st + 1);
-        if (st + 2 < nstep) step(std::integral_constant<int, 2>{}, st + 2);
-        if (st + 3 < nstep) step(std::integral_constant<int, 3>{}, st + 3);
+    for (int ch = 0; ch < nchunk; ch += 2) {               // nchunk is even: K a multiple of 2048
+        const uint4 sqn = *(const uint4*)(sp + min(ch + 2, nchunk - 1) / 2 * 16);
+        chunk(std::integral_constant<int, 0>{}, ch);
+        chunk(std::integral_constant<int, 1>{}, ch + 1);
         sq = sqn;
     }
     // D: lane = activation row c, output rows n0 + 4 g + i
@@ -674,11 +690,13 @@ SPARK_API int ds41_fp8_gemv_mx_q(const void* x, const void* aq, const void* as_,
 {
     if (m < 1 || m > 32 || k % 64 || n % 8 || (!x && !aq) || (aq && !as_)) return 1;
     if (k % 2048 == 0 && n % 16 == 0) {                    // the matrix unit: whole steps of 128 per K quarter, four at a time; whole 16-row tiles (each inside one 32-row scale group)
-        const auto need = [&](int rows) { return (size_t)rows * (k + FQ_CPAD) + (size_t)rows * (k / 32 + FQ_SPAD); };
-        const int per = need(16) <= 80 * 1024 ? 16 : need(8) <= 80 * 1024 ? 8 : 0;      // two workgroups per CU
+        const auto need = [&](int rows) { return (size_t)rows * (k + FQ_CPAD) + (size_t)rows * (k / 32 + FQ_SPAD) + 16 + 4 * 16 * FQ_TS; };
+        // rows per launch: 16 while two workgroups still share a CU (80 KB each); beyond that 16 for given codes, 8 when the kernel
+        // quantises (measured at 16 rows of 4096: 15.8 vs 17.9 us and 32.2 vs 28.5 us)
+        const int per = need(16) <= 80 * 1024 || (aq && need(16) <= 100 * 1024) ? 16 : need(8) <= 100 * 1024 ? 8 : 0;
         if (per) {
-            static bool attr = hipFuncSetAttribute((const void*)fp8q_mfma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) == hipSuccess &&
-                               hipFuncSetAttribute((const void*)fp8q_mfma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024) == hipSuccess;
+            static bool attr = hipFuncSetAttribute((const void*)fp8q_mfma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024) == hipSuccess &&
+                               hipFuncSetAttribute((const void*)fp8q_mfma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024) == hipSuccess;
             if (!attr) return 3;
             for (int r0 = 0; r0 < m; r0 += per) {
                 const int mm = m - r0 < per ? m - r0 : per;
