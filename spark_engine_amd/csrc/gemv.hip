@@ -392,11 +392,17 @@ __device__ __forceinline__ int wave_max_i(int v)
     v = max(v, __float_as_int(lane_xor<2>(__int_as_float(v), lane))); v = max(v, __float_as_int(lane_xor<1>(__int_as_float(v), lane)));
     return v;
 }
-template <int FMT, int KW>
+// TR: the weights are loaded as whole lines - one instruction reads 128 bytes of each of eight rows (lane l: row 8 i + l / 8,
+// bytes 16 (l % 8) of the chunk) - and a chunk goes through a wave-private LDS tile into the operand order; the 16-byte pieces
+// of 16 rows that the operand order asks of one instruction read a third slower (7168 x 4096 bytes: 9.0 vs 5.8 us).  Needs a
+// K part of whole chunks; other shapes load in operand order.
+constexpr int MG_CH = 128;             // bytes of a row per chunk
+constexpr int MG_TS = MG_CH + 16;      // row stride of a wave's transpose tile: 16-byte reads down its 16 rows hit distinct banks
+template <int FMT, int KW, bool TR>
 __global__ __launch_bounds__(64 * KW) void q_mfma_gemv_kernel(const uint16_t* __restrict__ x, int64_t xs, const uint8_t* __restrict__ w, const void* __restrict__ scv,
                                                           float* __restrict__ y, int m, int n, int k)
 {
-    extern __shared__ uint16_t xl[];                      // [m][k + MG_PAD] bf16
+    extern __shared__ uint16_t xl[];                      // [m][k + MG_PAD] bf16, then (TR) a tile of 16 x MG_TS bytes per wave
     __shared__ float red[KW][64][4];
     constexpr int NP = FMT == 0 ? 1 : 2;                  // 16-byte loads per piece
     constexpr int BPB = FMT == 0 ? 64 : 128;              // weight bytes of a row per 128-wide K block
@@ -408,20 +414,39 @@ __global__ __launch_bounds__(64 * KW) void q_mfma_gemv_kernel(const uint16_t* __
     const uint8_t* wp = w + (FMT == 0 ? (int64_t)row * (k / 2) + (kb0 + 32 * q) / 2 : (int64_t)row * k + kb0 + 32 * q);
     const float* spf = (const float*)scv + (int64_t)(n0 / 128) * sld + kb0 / 128;                                  // FMT 2: one per block
     const uint8_t* spb = (const uint8_t*)scv + (int64_t)(FMT == 1 ? row / 32 : row) * (k / 32) + kb0 / 32 + q;     // E8M0: one per piece
-    // the first four K blocks are on their way before the activations are staged
+    // the first four K blocks (TR: four chunks) are on their way before the activations are staged
+    constexpr int BPC = MG_CH / BPB;                      // K blocks per chunk (TR)
     uint4 p[4][NP];
-    float s2[4];
-    uint32_t sb[4];
-    auto fetch = [&](auto uc, int b) {
+    uint4 pc[4][2];                                       // TR: chunk u, rows 8 i + lane / 8
+    float s2[4], s2c[4][BPC];
+    uint32_t sb[4], sbc[4][BPC];
+    const int lr = lane >> 3, lc = (lane & 7) * 16, nchunk = nblk / BPC;
+    const uint8_t* wpc = w + (int64_t)(n0 + lr) * (FMT == 0 ? k / 2 : k) + (FMT == 0 ? kb0 / 2 : kb0) + lc;
+    unsigned char* tw = (unsigned char*)xl + (((size_t)m * ld * 2 + 15) & ~(size_t)15) + (size_t)wave * (16 * MG_TS);
+    auto fetch = [&](auto uc, int b) {                    // operand order: block b into ring slot u
         constexpr int u = decltype(uc)::value;
 #pragma unroll
         for (int h = 0; h < NP; ++h) p[u][h] = ld_stream16(wp + b * BPB + h * 16);
         if constexpr (FMT == 2) s2[u] = spf[b]; else sb[u] = spb[b * 4];
     };
-    fetch(std::integral_constant<int, 0>{}, 0);
-    fetch(std::integral_constant<int, 1>{}, min(1, nblk - 1));
-    fetch(std::integral_constant<int, 2>{}, min(2, nblk - 1));
-    fetch(std::integral_constant<int, 3>{}, min(3, nblk - 1));
+    auto fetch_chunk = [&](auto uc, int ch) {             // TR: chunk ch and its blocks' scales into ring slot u
+        constexpr int u = decltype(uc)::value;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) pc[u][i] = ld_stream16(wpc + (int64_t)(8 * i) * (FMT == 0 ? k / 2 : k) + ch * MG_CH);
+#pragma unroll
+        for (int j = 0; j < BPC; ++j) { if constexpr (FMT == 2) s2c[u][j] = spf[ch * BPC + j]; else sbc[u][j] = spb[(ch * BPC + j) * 4]; }
+    };
+    if constexpr (TR) {
+        fetch_chunk(std::integral_constant<int, 0>{}, 0);
+        fetch_chunk(std::integral_constant<int, 1>{}, min(1, nchunk - 1));
+        fetch_chunk(std::integral_constant<int, 2>{}, min(2, nchunk - 1));
+        fetch_chunk(std::integral_constant<int, 3>{}, min(3, nchunk - 1));
+    } else {
+        fetch(std::integral_constant<int, 0>{}, 0);
+        fetch(std::integral_constant<int, 1>{}, min(1, nblk - 1));
+        fetch(std::integral_constant<int, 2>{}, min(2, nblk - 1));
+        fetch(std::integral_constant<int, 3>{}, min(3, nblk - 1));
+    }
     {
         const int n8 = k / 8;
         for (int i = threadIdx.x; i < m * n8; i += 64 * KW) {
@@ -432,21 +457,20 @@ __global__ __launch_bounds__(64 * KW) void q_mfma_gemv_kernel(const uint16_t* __
     __syncthreads();
     const uint16_t* xr = xl + min(c, m - 1) * ld + kb0 + 32 * q;
     v4f tot = v4f{0.f, 0.f, 0.f, 0.f};
-    auto step = [&](auto uc, int b) {
-        constexpr int u = decltype(uc)::value;
+    auto mma_block = [&](const uint4 (&pp)[NP], int b, float s2v, uint32_t sbv) {
         v4f cur = v4f{0.f, 0.f, 0.f, 0.f};
         float cs = 1.0f, sv;
-        if constexpr (FMT == 2) sv = s2[u];
+        if constexpr (FMT == 2) sv = s2v;
         else {
-            const int top = wave_max_i((int)sb[u]);
-            cs = __uint_as_float((uint32_t)max((int)sb[u] - top + 127, 0) << 23);
+            const int top = wave_max_i((int)sbv);
+            cs = __uint_as_float((uint32_t)max((int)sbv - top + 127, 0) << 23);
             sv = e8m0_to_f32((uint32_t)top);
         }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             bf2 wv[8];
             if constexpr (FMT == 0) {
-                const uint32_t pw[2] = {h ? p[u][0].z : p[u][0].x, h ? p[u][0].w : p[u][0].y};
+                const uint32_t pw[2] = {h ? pp[0].z : pp[0].x, h ? pp[0].w : pp[0].y};
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     wv[4 * j + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], cs, 0);
@@ -455,7 +479,7 @@ __global__ __launch_bounds__(64 * KW) void q_mfma_gemv_kernel(const uint16_t* __
                     wv[4 * j + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(pw[j], cs, 3);
                 }
             } else {
-                const uint4 pv = p[u][NP - 1 < h ? NP - 1 : h];
+                const uint4 pv = pp[NP - 1 < h ? NP - 1 : h];
                 const uint32_t pw[4] = {pv.x, pv.y, pv.z, pv.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -470,15 +494,54 @@ __global__ __launch_bounds__(64 * KW) void q_mfma_gemv_kernel(const uint16_t* __
             cur = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, cur, 0, 0, 0);
             cur = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, cur, 0, 0, 0);
         }
-        fetch(uc, min(b + 4, nblk - 1));                  // four blocks ahead, into the registers just used
 #pragma unroll
         for (int i = 0; i < 4; ++i) tot[i] = __builtin_fmaf(cur[i], sv, tot[i]);
     };
-    for (int b = 0; b < nblk; b += 4) {
-        step(std::integral_constant<int, 0>{}, b);
-        if (b + 1 < nblk) step(std::integral_constant<int, 1>{}, b + 1);
-        if (b + 2 < nblk) step(std::integral_constant<int, 2>{}, b + 2);
-        if (b + 3 < nblk) step(std::integral_constant<int, 3>{}, b + 3);
+    auto step = [&](auto uc, int b) {
+        constexpr int u = decltype(uc)::value;
+        uint4 pp[NP];
+#pragma unroll
+        for (int h = 0; h < NP; ++h) pp[h] = p[u][h];
+        const float s2v = s2[u];
+        const uint32_t sbv = sb[u];
+        fetch(uc, min(b + 4, nblk - 1));                  // four blocks ahead, into the registers just used
+        mma_block(pp, b, s2v, sbv);
+    };
+    auto chunk = [&](auto uc, int ch) {
+        constexpr int u = decltype(uc)::value;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *(uint4*)(tw + (8 * i + lr) * MG_TS + lc) = pc[u][i];
+        __builtin_amdgcn_wave_barrier();                   // the tile belongs to this wave: its LDS operations execute in order
+        asm volatile("" ::: "memory");
+        uint4 q4[BPC][NP];
+#pragma unroll
+        for (int j = 0; j < BPC; ++j)
+#pragma unroll
+            for (int h = 0; h < NP; ++h) q4[j][h] = *(const uint4*)(tw + c * MG_TS + j * BPB + (FMT == 0 ? 16 : 32) * q + h * 16);
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+        float s2l[BPC];
+        uint32_t sbl[BPC];
+#pragma unroll
+        for (int j = 0; j < BPC; ++j) { s2l[j] = s2c[u][j]; sbl[j] = sbc[u][j]; }
+        fetch_chunk(uc, min(ch + 4, nchunk - 1));          // four chunks ahead, into the registers just used
+#pragma unroll
+        for (int j = 0; j < BPC; ++j) mma_block(q4[j], ch * BPC + j, s2l[j], sbl[j]);
+    };
+    if constexpr (TR) {
+        for (int ch = 0; ch < nchunk; ch += 4) {
+            chunk(std::integral_constant<int, 0>{}, ch);
+            if (ch + 1 < nchunk) chunk(std::integral_constant<int, 1>{}, ch + 1);
+            if (ch + 2 < nchunk) chunk(std::integral_constant<int, 2>{}, ch + 2);
+            if (ch + 3 < nchunk) chunk(std::integral_constant<int, 3>{}, ch + 3);
+        }
+    } else {
+        for (int b = 0; b < nblk; b += 4) {
+            step(std::integral_constant<int, 0>{}, b);
+            if (b + 1 < nblk) step(std::integral_constant<int, 1>{}, b + 1);
+            if (b + 2 < nblk) step(std::integral_constant<int, 2>{}, b + 2);
+            if (b + 3 < nblk) step(std::integral_constant<int, 3>{}, b + 3);
+        }
     }
     // D: lane = activation row c, output rows n0 + 4 q + i
 #pragma unroll
@@ -630,14 +693,31 @@ int launch_qgemv(const void* x, const void* w, const void* sc, float* y, int m, 
     if (m >= 3 && k % 512 == 0 && n % 16 == 0 && rpg == 0 && (FMT != 2 || bs == 128)) {     // three or more rows: the matrix unit
         const size_t smm = (size_t)m * (k + MG_PAD) * 2;
         if (smm <= MFMA_LDS_MAX) {
-            static bool attr = hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess &&
-                               hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess;
+            static bool attr = hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 4, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess &&
+                               hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 8, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess &&
+                               hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 4, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess &&
+                               hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 7, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess &&
+                               hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 8, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess;
             if (!attr) return 3;
+            // whole-line loads when a K part is whole chunks of 128 bytes a row: in eighths or sevenths for matrices whose row tiles
+            // leave a CU one workgroup, else in quarters
+            {
+                const int cel = FMT == 0 ? 256 : 128;     // k per chunk
+                const size_t tile = (size_t)16 * MG_TS;
+                const int kw = n / 16 <= 256 && k % (8 * cel) == 0 ? 8 : n / 16 <= 256 && k % (7 * cel) == 0 ? 7 : k % (4 * cel) == 0 ? 4 : 0;
+                const size_t smt = ((smm + 15) & ~(size_t)15) + kw * tile;
+                if (kw && smt <= MFMA_LDS_MAX) {
+                    if (kw == 8) q_mfma_gemv_kernel<FMT, 8, true><<<n / 16, 512, smt, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
+                    else if (kw == 7) q_mfma_gemv_kernel<FMT, 7, true><<<n / 16, 448, smt, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
+                    else q_mfma_gemv_kernel<FMT, 4, true><<<n / 16, 256, smt, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
+                    return launch_status();
+                }
+            }
             // K in quarters, or in eighths when the row tiles leave a CU with a single workgroup and an eighth is still six K blocks
             // or more (4096 x 7168 at 4 rows: 13.5 -> 12.0 us; 7168 x 4096 in eighths: 11.9 -> 16.2 us).  The split depends on the
             // shape only: a row's value does not depend on the row count
-            if (n / 16 <= 256 && k % 1024 == 0 && k >= 6144) q_mfma_gemv_kernel<FMT, 8><<<n / 16, 512, smm, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
-            else q_mfma_gemv_kernel<FMT, 4><<<n / 16, 256, smm, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
+            if (n / 16 <= 256 && k % 1024 == 0 && k >= 6144) q_mfma_gemv_kernel<FMT, 8, false><<<n / 16, 512, smm, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
+            else q_mfma_gemv_kernel<FMT, 4, false><<<n / 16, 256, smm, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
             return launch_status();
         }
     }
