@@ -190,6 +190,19 @@ def test_matrix_unit_gemvs(ops, oracle, m, n, k):
         assert np.array_equal(ys, y[:sub])
 
 
+def test_bf16_gemv_tall_matrix_rows(ops):
+    # three or more rows of a tall matrix take the row-tile kernel, four rows per launch
+    g = synth.rng(170)
+    n, k, m = 8192, 1024, 7
+    wb = synth.randn_bf16(g, (n, k))
+    x = synth.randn_bf16(g, (m, k))
+    y = host(ops.bf16_gemv(dev_bf16(x), dev_bf16(wb)))
+    ref = synth.bf16_to_f32(x).astype(np.float64) @ synth.bf16_to_f32(wb).astype(np.float64).T
+    assert rel_l2(y, ref) < 1e-5
+    y3 = host(ops.bf16_gemv(dev_bf16(x[:3]), dev_bf16(wb)))
+    assert np.array_equal(y3, y[:3])
+
+
 def test_fp8_gemv_bx_up_to_16_rows_and_groups(ops, oracle):
     g = synth.rng(150)
     n, k, m = 256, 512, 13
