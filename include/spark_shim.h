@@ -40,7 +40,7 @@ SPARK_API int spark_exl3_fold(const void* trellis, const void* suh, const void* 
 SPARK_API int qwen_exl3_fold(const void* trellis, const void* suh, const void* svh, int K, int N, int bits, void* out_f16, int64_t ldo,
                              hipStream_t st);
 /* Dense EXL3 linears for M <= 64 rows, trellis widths 3..6 bits, mul1 codebook: y = had128(had128(x * suh) @ inner) * svh in three
- * steps or at once.  xh [M, K] fp16, part [S, M, N] fp32 (S = K slices, summed in order), cnt unused.  qwen_exl3_multi: up to 4
+ * steps or at once.  xh [M, K] fp16, part [S, M, N] fp32 (S = K slices, summed in order), cnt unused (may be NULL; left as it is).  qwen_exl3_multi: up to 4
  * linears on the same x (silu bit 0 with n = 2: y[0] = silu(linear 0) * linear 1); with mg / mn (fp32 [M, 4, K]) the input is
  * (1/4) sum_s mn[m][s][k] * sigmoid(mg[m][s][k]), also written to xout fp32 [M, K]; silu bits 1 and 2 (separate launches, fork
  * onto the reference runtime's side stream) are accepted and change nothing here: everything runs on st.

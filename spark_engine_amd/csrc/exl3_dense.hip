@@ -109,6 +109,89 @@ __global__ __launch_bounds__(DT) void dense_gemv_kernel(const void* __restrict__
     }
 }
 
+// The 4-bit case of the product above, the width every decode-time projection of the reference models has: the weight stream and
+// decode of the expert kernels.  grid (N / 128, S), 8 waves; a wave reads eight consecutive tiles of a k-tile row (1 KB) with one
+// 16-byte load per lane, four k-tiles in flight, decodes its 2 columns x 16 k per tile in registers and multiplies with
+// v_dot2_f32_f16 against the transformed rows in LDS; the waves' sums are added in wave order.  Up to 8 rows.
+constexpr int D4_WAVES = 8, D4_FLY = 4;
+template <int CBK, int MR>
+__device__ __forceinline__ void tile_fma4(const uint4 w, uint32_t prev, const uint32_t* xrow, int ldx32, int rows, float (&acc)[MR][2])
+{
+    h2 wd[4][4];
+    decode_tile32<CBK>(w, prev, wd);
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+        if (r >= rows) break;
+        dot_tile32(wd, xrow + r * ldx32, acc[r][0], acc[r][1]);   // 8 packed fp16 pairs of this k-tile (wave-uniform address)
+    }
+}
+template <int CBK, int MR, int XMODE>
+__global__ __launch_bounds__(64 * D4_WAVES) void dense4_gemv_kernel(const void* __restrict__ xin, int64_t ldx, const uint16_t* __restrict__ suh,
+                                                                    const uint32_t* __restrict__ tr, float* __restrict__ part, int M, int K, int N, int kts, int kpad)
+{
+    extern __shared__ __align__(16) unsigned char sm[];
+    __shared__ float red[D4_WAVES][MR][128];
+    const int Kt = K / 16, Nt = N / 16;
+    const int nb = blockIdx.x, s = blockIdx.y;
+    const int kt0 = s * kts, kt1 = min(Kt, kt0 + kts);
+    uint16_t* xs = (uint16_t*)sm;                                          // [M][kpad] fp16 of the transformed rows from k0 on
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int k0 = kt0 * 16 / 128 * 128;                                   // first Hadamard block touching the slice
+    const int off = kt0 * 16 - k0;
+    const int src = tile_prev_lane(lane);
+    // the wave's first k-tiles are on their way before the rows are staged
+    uint4 wt[D4_FLY];
+#pragma unroll
+    for (int u = 0; u < D4_FLY; ++u) {
+        const int kt = min(min(kt0 + wave + u * D4_WAVES, max(kt1 - 1, kt0)), Kt - 1);   // an empty slice (more slices than k-tiles) reads a valid tile and uses nothing
+        wt[u] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
+    }
+    if (XMODE == 0) {
+        for (int i = tid; i < M * (kpad / 2); i += 64 * D4_WAVES) {
+            const int r = i / (kpad / 2), c = (i % (kpad / 2)) * 2;
+            *(uint32_t*)(xs + (size_t)r * kpad + c) = k0 + c < K ? *(const uint32_t*)((const uint16_t*)xin + (int64_t)r * K + k0 + c) : 0u;
+        }
+    } else {
+        const int nblk = kpad / 128;
+        for (int u = wave; u < M * nblk; u += D4_WAVES) {
+            const int r = u / nblk, k = k0 + (u % nblk) * 128 + 2 * lane;
+            float v0 = 0.f, v1 = 0.f;
+            if (k < K) {
+                v0 = ((const float*)xin)[r * ldx + k] * f16_bits_to_f32(suh[k]);
+                v1 = ((const float*)xin)[r * ldx + k + 1] * f16_bits_to_f32(suh[k + 1]);
+            }
+            fwht128(v0, v1, lane);
+            *(uint32_t*)(xs + (size_t)r * kpad + (k - k0)) = (uint32_t)f32_to_f16_bits(v0) | ((uint32_t)f32_to_f16_bits(v1) << 16);
+        }
+    }
+    __syncthreads();
+    const uint32_t* xbase = (const uint32_t*)(xs + off);                  // k-tile kt of row r: xbase + r * kpad / 2 + (kt - kt0) * 8
+    float acc[MR][2];
+#pragma unroll
+    for (int r = 0; r < MR; ++r) { acc[r][0] = 0.f; acc[r][1] = 0.f; }
+    for (int kt = kt0 + wave; kt < kt1; kt += D4_FLY * D4_WAVES) {
+#pragma unroll
+        for (int u = 0; u < D4_FLY; ++u) {
+            const int ktu = kt + u * D4_WAVES;
+            const uint4 w = wt[u];
+            const int ktn = min(ktu + D4_FLY * D4_WAVES, kt1 - 1);        // the same slot of the next round (past the end: a tile again, unused)
+            wt[u] = ld_stream16(tr + ((int64_t)ktn * Nt + nb * 8) * 32 + lane * 4);
+            if (ktu < kt1) tile_fma4<CBK, MR>(w, __shfl(w.w, src, 64), xbase + (ktu - kt0) * 8, kpad / 2, M, acc);
+        }
+    }
+    const int j = lane >> 3, mm = lane & 7;
+#pragma unroll
+    for (int r = 0; r < MR; ++r) { red[wave][r][16 * j + mm] = acc[r][0]; red[wave][r][16 * j + mm + 8] = acc[r][1]; }
+    __syncthreads();
+    for (int i = tid; i < M * 128; i += 64 * D4_WAVES) {
+        const int r = i >> 7, c = i & 127;
+        float v = red[0][r][c];
+#pragma unroll
+        for (int w = 1; w < D4_WAVES; ++w) v += red[w][r][c];
+        part[((int64_t)s * M + r) * N + nb * 128 + c] = v;
+    }
+}
+
 // y[m, n] = had128(sum_s part[s][m][:]) * svh (the silu form: y = silu(linear 0) * linear 1); one wave per (row, 128-block)
 template <bool PH, bool YF32>
 __global__ __launch_bounds__(256) void finish_kernel(const void* __restrict__ part, int S, const uint16_t* __restrict__ svh, void* __restrict__ y, int64_t ldy,
@@ -148,6 +231,20 @@ int launch_gemv(int xmode, const void* x, int64_t ldx, const void* suh, const vo
     const size_t smem = (size_t)M * kpad * 2 + 16 * 128 * 2 + 8 * 48 * 4;
     if (smem > 160 * 1024) return -1;
     const dim3 grid(N / 128, S);
+    if (bits == 4 && M <= 8) {
+        const size_t sm4 = (size_t)M * kpad * 2;
+#define D4(CB, MRR)                                                                                                                             \
+    do {                                                                                                                                        \
+        if (xmode) dense4_gemv_kernel<CB, MRR, 1><<<grid, 64 * D4_WAVES, sm4, st>>>(x, ldx, (const uint16_t*)suh, (const uint32_t*)trellis, (float*)part, M, K, N, kts, kpad); \
+        else dense4_gemv_kernel<CB, MRR, 0><<<grid, 64 * D4_WAVES, sm4, st>>>(x, ldx, (const uint16_t*)suh, (const uint32_t*)trellis, (float*)part, M, K, N, kts, kpad);       \
+    } while (0)
+        if (sm4 <= 48 * 1024) {
+            if (codebook == CB_MCG) { if (M == 1) D4(CB_MCG, 1); else if (M == 2) D4(CB_MCG, 2); else if (M <= 4) D4(CB_MCG, 4); else D4(CB_MCG, 8); }
+            else { if (M == 1) D4(CB_MUL1, 1); else if (M == 2) D4(CB_MUL1, 2); else if (M <= 4) D4(CB_MUL1, 4); else D4(CB_MUL1, 8); }
+            return launch_status();
+        }
+#undef D4
+    }
 #define DG(CB, XM)                                                                                                                              \
     do {                                                                                                                                        \
         static bool attr = hipFuncSetAttribute((const void*)dense_gemv_kernel<CB, XM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess; \
@@ -206,7 +303,9 @@ SPARK_API int qwen_exl3_finish_h(const void* part, const void* svh, void* y, int
     finish_kernel<true, true><<<blocks, 256, 0, st>>>(part, 1, (const uint16_t*)svh, y, ldy, M, N, nullptr, nullptr);
     return launch_status();
 }
-// x [M <= 64, K] fp32 -> y [M, N] fp32; part: scratch [S, M, N] fp32; cnt is not used here (two launches, no counters).
+// x [M <= 64, K] fp32 -> y [M, N] fp32; part: scratch [S, M, N] fp32; cnt is not used: two launches (product, finish).  Finishing
+// inside the product's launch behind per-column-block counters, as the reference does, was measured slower here (2560 -> 512:
+// 10.6 vs 8.1 us, 640 -> 2560: 18.5 vs 6.2 us: every workgroup pays a device-wide fence before its count).
 // reference qwen_exl3.cu:150-168
 SPARK_API int qwen_exl3_linear(const void* x, int64_t ldx, const void* suh, const void* trellis, const void* svh, void* part, void* y, int64_t ldy, void* cnt,
                                int M, int K, int N, int bits, int S, hipStream_t st)

@@ -80,15 +80,19 @@ def exl3_finish(part, svh, f32=True):
     return y
 
 
-def exl3_linear(x, suh, trellis, svh, S=4):
-    """x f32 [M, K] -> y f32 [M, N] (had_in + gemv + finish)."""
+def exl3_linear(x, suh, trellis, svh, S=4, counters=False):
+    """x f32 [M, K] -> y f32 [M, N] (had_in + gemv + finish).  counters: hand the entry point its counter array (one launch
+    where it can); returns (y, cnt)."""
     M, K = x.shape
     Kt, Nt, W = trellis.shape
     N = Nt * 16
     part = torch.empty(S, M, N, dtype=torch.float32, device=x.device)
     y = torch.empty(M, N, dtype=torch.float32, device=x.device)
-    _ck(_lib().qwen_exl3_linear(_p(x), x.stride(0), _p(_dev(suh)), _p(_dev(trellis)), _p(_dev(svh)), _p(part), _p(y), N, None, M, K, N, W // 16, S, _st()),
+    cnt = torch.zeros(N // 128, dtype=torch.int32, device=x.device) if counters else None      # zero before, zero after (reference qwen_exl3.cu:148-149)
+    _ck(_lib().qwen_exl3_linear(_p(x), x.stride(0), _p(_dev(suh)), _p(_dev(trellis)), _p(_dev(svh)), _p(part), _p(y), N, _p(cnt), M, K, N, W // 16, S, _st()),
         "qwen_exl3_linear")
+    if counters:
+        return y, cnt
     return y
 
 

@@ -49,12 +49,29 @@ def test_linear_steps_and_fused_form(ops, oracle, bits):
     assert rel_l2(y, ref) <= 1e-3, rel_l2(y, ref)
     y2 = host(ops.exl3_linear(dev(x), dev_f16(suh), dev(tr), dev_f16(svh), S=S))
     assert np.array_equal(y, y2)                                         # the one-call form does the same arithmetic
+    y3, cnt = ops.exl3_linear(dev(x), dev_f16(suh), dev(tr), dev_f16(svh), S=S, counters=True)
+    assert np.array_equal(y, host(y3)) and int(cnt.abs().sum().item()) == 0            # a counter array handed in stays zero
     yh = host(ops.exl3_finish(part, dev_f16(svh), f32=False)).view(np.float16).astype(np.float32)
     assert np.array_equal(yh, y.astype(np.float16).astype(np.float32))
     x16 = x.astype(np.float16)
     xh16 = ops.exl3_had_in(dev_f16(x16.view(np.uint16)), dev_f16(suh))  # fp16 input form
     _, xh_ref16 = _reference(oracle, x16.astype(np.float32), tr, suh, svh)
     assert np.array_equal(host(xh16).view(np.float16).astype(np.float32), xh_ref16)
+
+
+def test_linear_decode_shapes(ops, oracle):
+    # the reference's published GEMV shapes (2560 -> 512, 640 -> 2560), one row, 4 bits: the fast 4-bit kernel, K slices that do not
+    # divide the k-tiles evenly included
+    g = synth.rng(505)
+    for K, N, S in ((2560, 512, 4), (640, 2560, 4), (640, 256, 3), (256, 128, 7)):
+        tr, suh, svh = synth.exl3_matrix(g, K, N, 4)
+        for M in (1, 3, 8):
+            x = g.standard_normal((M, K)).astype(np.float32)
+            ref, _ = _reference(oracle, x, tr, suh, svh)
+            y = host(ops.exl3_linear(dev(x), dev_f16(suh), dev(tr), dev_f16(svh), S=S))
+            assert rel_l2(y, ref) <= 1e-3, (K, N, S, M, rel_l2(y, ref))
+            y1 = host(ops.exl3_linear(dev(x[:1]), dev_f16(suh), dev(tr), dev_f16(svh), S=S))
+            assert np.array_equal(y1[0], y[0])                            # a row's value does not depend on the row count
 
 
 def test_multi_and_silu(ops, oracle):
