@@ -634,25 +634,26 @@ __global__ __launch_bounds__(64 * KW) void q_mfma_gemv_kernel(const uint16_t* __
 
 // The same product on the matrix unit: v_mfma_scale_f32_16x16x128_f8f6f4 multiplies E4M3 by E4M3 with an E8M0 scale per 32 k on
 // either side, which is this format exactly (the products and scales are exact, the sums binary32).  Workgroup = 16 weight rows,
-// wave = a quarter of K; a lane's A operand of a 128-wide step is 16 bytes at k = 16 g and 16 at 64 + 16 g of its row, two
+// wave = one of 1-8 equal parts of K (quarters where K allows); a lane's A operand of a 128-wide step is 16 bytes at k = 16 g and 16 at 64 + 16 g of its row, two
 // chunks of 256 k in flight; the activation codes and scales (given, or quantised here by the rule of act_quant) sit in LDS with
 // row strides that spread the 16 rows over the banks.  Up to 16 activation rows per launch: the columns of the tile.  The four
-// K quarters are summed through LDS in wave order.  A row's value does not depend on the rows beside it.
+// K parts are summed through LDS in wave order.  A row's value does not depend on the rows beside it.
 constexpr int FQ_CPAD = 16, FQ_SPAD = 4;
 constexpr int FQ_TS = 256 + 16;        // row stride of a wave's transpose tile: 16-byte reads down its 16 rows hit distinct banks
-template <bool QUANT>
-__global__ __launch_bounds__(256) void fp8q_mfma_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ aq, const uint8_t* __restrict__ as_,
+template <bool QUANT, int NW>                          // NW: waves = K parts at compile time, or 0: from the launch (up to 8)
+__global__ __launch_bounds__(NW ? 64 * NW : 512) void fp8q_mfma_kernel(const uint16_t* __restrict__ x, const uint8_t* __restrict__ aq, const uint8_t* __restrict__ as_,
                                                         const uint8_t* __restrict__ w, const uint8_t* __restrict__ ws, void* __restrict__ y, int ob16, int m, int n,
                                                         int k)
 {
     extern __shared__ __align__(16) unsigned char fq_lds[];
-    __shared__ float red[4][64][4];
+    __shared__ float red[8][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
+    const int nw = NW ? NW : (int)(blockDim.x >> 6), nthr = 64 * nw;
     const int cld = k + FQ_CPAD, nb32 = k >> 5, sld = nb32 + FQ_SPAD;
     unsigned char* xc = fq_lds;                           // [m][k + pad] codes
     unsigned char* xs = fq_lds + (size_t)m * cld;         // [m][k / 32 + pad] scale bytes
     const int n0 = blockIdx.x * 16;
-    const int ks = k / 4, kb0 = wave * ks, nstep = ks / 128;
+    const int ks = k / nw, kb0 = wave * ks, nstep = ks / 128;       // a K part is whole chunks of 256
     // Weight loads: one instruction reads 256 bytes of each of four rows (lane l: row 4 i + l / 16, bytes 16 (l % 16) of the
     // chunk), whole lines side by side - 64-byte pieces of 16 rows per instruction, the operand's own order, read a third slower.
     // The chunk goes through a wave-private LDS tile into the operand order (lane = row c, K block g).
@@ -660,17 +661,18 @@ __global__ __launch_bounds__(256) void fp8q_mfma_kernel(const uint16_t* __restri
     const uint8_t* wp = w + (int64_t)(n0 + lr) * k + kb0 + lc;
     unsigned char* tw = fq_lds + (((size_t)m * cld + (size_t)m * sld + 15) & ~(size_t)15) + (size_t)wave * (16 * FQ_TS);
     const uint8_t* sp = ws + (int64_t)(n0 >> 5) * nb32 + kb0 / 32;        // the tile's 16 rows share a 32-row scale group
-    uint4 a[2][4], sq;
+    uint4 a[2][4];
+    uint2 sq[2];                                          // the scale bytes of a chunk's two steps (8 blocks), the same for every lane
     auto fetch = [&](auto uc, int ch) {
         constexpr int u = decltype(uc)::value;
 #pragma unroll
         for (int i = 0; i < 4; ++i) a[u][i] = ld_stream16(wp + (int64_t)(4 * i) * k + ch * 256);
+        sq[u] = *(const uint2*)(sp + ch * 8);
     };
     fetch(std::integral_constant<int, 0>{}, 0);
     fetch(std::integral_constant<int, 1>{}, min(1, nchunk - 1));
-    sq = *(const uint4*)sp;                                // the scale bytes of four steps (16 blocks), the same for every lane
     if (QUANT) {
-        for (int i = threadIdx.x; i < m * nb32 * 4; i += 256) {            // 4 threads per 32-block, 8 elements each
+        for (int i = threadIdx.x; i < m * nb32 * 4; i += nthr) {           // 4 threads per 32-block, 8 elements each
             const int r = i / (nb32 * 4), q = i % (nb32 * 4), b = q >> 2, col = b * 32 + (q & 3) * 8;
             const uint4 raw = *(const uint4*)(x + (int64_t)r * k + col);
             const uint32_t rw4[4] = {raw.x, raw.y, raw.z, raw.w};
@@ -688,11 +690,11 @@ __global__ __launch_bounds__(256) void fp8q_mfma_kernel(const uint16_t* __restri
         }
     } else {
         const int n16 = k / 16;
-        for (int i = threadIdx.x; i < m * n16; i += 256) {
+        for (int i = threadIdx.x; i < m * n16; i += nthr) {
             const int r = i / n16, col = (i % n16) * 16;
             *(uint4*)(xc + (size_t)r * cld + col) = *(const uint4*)(aq + (int64_t)r * k + col);
         }
-        for (int i = threadIdx.x; i < m * (nb32 / 4); i += 256) {
+        for (int i = threadIdx.x; i < m * (nb32 / 4); i += nthr) {
             const int r = i / (nb32 / 4), col = (i % (nb32 / 4)) * 4;
             *(uint32_t*)(xs + r * sld + col) = *(const uint32_t*)(as_ + (int64_t)r * nb32 + col);
         }
@@ -713,6 +715,7 @@ __global__ __launch_bounds__(256) void fp8q_mfma_kernel(const uint16_t* __restri
         for (int s2 = 0; s2 < 2; ++s2) { al[s2][0] = *(const uint4*)(tw + c * FQ_TS + s2 * 128 + 16 * g); al[s2][1] = *(const uint4*)(tw + c * FQ_TS + s2 * 128 + 64 + 16 * g); }
         __builtin_amdgcn_wave_barrier();
         asm volatile("" ::: "memory");
+        const uint2 sqc = sq[u];
         fetch(uc, min(ch + 2, nchunk - 1));                // two chunks ahead, into the registers just used
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
@@ -720,17 +723,15 @@ __global__ __launch_bounds__(256) void fp8q_mfma_kernel(const uint16_t* __restri
             const uint4 lo = *(const uint4*)(bc + st * 128), hi = *(const uint4*)(bc + st * 128 + 64);
             const v8i b8 = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
             const v8i a8 = v8i{(int)al[s2][0].x, (int)al[s2][0].y, (int)al[s2][0].z, (int)al[s2][0].w, (int)al[s2][1].x, (int)al[s2][1].y, (int)al[s2][1].z, (int)al[s2][1].w};
-            const uint32_t sdw = u == 0 ? (s2 ? sq.y : sq.x) : (s2 ? sq.w : sq.z);
+            const uint32_t sdw = s2 ? sqc.y : sqc.x;
             const uint32_t sa = (sdw >> (8 * g)) & 0xffu;
             const uint32_t sb = (*(const uint32_t*)(bs + st * 4) >> (8 * g)) & 0xffu;
             acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc, 0 /*A: E4M3*/, 0 /*B: E4M3*/, 0, (int)sa, 0, (int)sb);
         }
     };
-    for (int ch = 0; ch < nchunk; ch += 2) {               // nchunk is even: K a multiple of 2048
-        const uint4 sqn = *(const uint4*)(sp + min(ch + 2, nchunk - 1) / 2 * 16);
+    for (int ch = 0; ch < nchunk; ch += 2) {
         chunk(std::integral_constant<int, 0>{}, ch);
-        chunk(std::integral_constant<int, 1>{}, ch + 1);
-        sq = sqn;
+        if (ch + 1 < nchunk) chunk(std::integral_constant<int, 1>{}, ch + 1);
     }
     // D: lane = activation row c, output rows n0 + 4 g + i
 #pragma unroll
@@ -739,7 +740,8 @@ __global__ __launch_bounds__(256) void fp8q_mfma_kernel(const uint16_t* __restri
     if (wave == 0 && c < m) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float v = ((red[0][lane][i] + red[1][lane][i]) + red[2][lane][i]) + red[3][lane][i];
+            float v = red[0][lane][i];
+            for (int u = 1; u < nw; ++u) v += red[u][lane][i];
             const int64_t o = (int64_t)c * n + n0 + 4 * g + i;
             if (ob16) ((uint16_t*)y)[o] = f32_to_bf16(v); else ((float*)y)[o] = v;
         }
@@ -843,22 +845,32 @@ SPARK_API int ds41_fp8_gemv_mx_q(const void* x, const void* aq, const void* as_,
                                  hipStream_t st)
 {
     if (m < 1 || m > 32 || k % 64 || n % 8 || (!x && !aq) || (aq && !as_)) return 1;
-    if (k % 2048 == 0 && n % 16 == 0) {                    // the matrix unit: whole steps of 128 per K quarter, four at a time; whole 16-row tiles (each inside one 32-row scale group)
-        const auto need = [&](int rows) { return (size_t)rows * (k + FQ_CPAD) + (size_t)rows * (k / 32 + FQ_SPAD) + 16 + 4 * 16 * FQ_TS; };
+    // the matrix unit: whole 16-row tiles (each inside one 32-row scale group), K in nw parts of whole 256-wide chunks: quarters
+    // where they are, else the most parts up to 8 (1280 -> 5, 3072 -> 6)
+    int nw = 0;
+    if (k % 1024 == 0) nw = 4;
+    else for (int t = 8; t >= 1 && !nw; --t) if (k % (t * 256) == 0) nw = t;
+    if (nw && n % 16 == 0) {
+        const auto need = [&](int rows) { return (size_t)rows * (k + FQ_CPAD) + (size_t)rows * (k / 32 + FQ_SPAD) + 16 + (size_t)nw * 16 * FQ_TS; };
         // rows per launch: 16 while two workgroups still share a CU (80 KB each); beyond that 16 for given codes, 8 when the kernel
         // quantises (measured at 16 rows of 4096: 15.8 vs 17.9 us and 32.2 vs 28.5 us)
         const int per = need(16) <= 80 * 1024 || (aq && need(16) <= 100 * 1024) ? 16 : need(8) <= 100 * 1024 ? 8 : 0;
         if (per) {
-            static bool attr = hipFuncSetAttribute((const void*)fp8q_mfma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024) == hipSuccess &&
-                               hipFuncSetAttribute((const void*)fp8q_mfma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024) == hipSuccess;
+            static bool attr = hipFuncSetAttribute((const void*)fp8q_mfma_kernel<true, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024) == hipSuccess &&
+                               hipFuncSetAttribute((const void*)fp8q_mfma_kernel<false, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024) == hipSuccess &&
+                               hipFuncSetAttribute((const void*)fp8q_mfma_kernel<true, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024) == hipSuccess &&
+                               hipFuncSetAttribute((const void*)fp8q_mfma_kernel<false, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024) == hipSuccess;
             if (!attr) return 3;
             for (int r0 = 0; r0 < m; r0 += per) {
                 const int mm = m - r0 < per ? m - r0 : per;
                 void* yr = ob16 ? (void*)((uint16_t*)y + (int64_t)r0 * n) : (void*)((float*)y + (int64_t)r0 * n);
-                if (aq) fp8q_mfma_kernel<false><<<n / 16, 256, need(mm), st>>>(nullptr, (const uint8_t*)aq + (int64_t)r0 * k, (const uint8_t*)as_ + (int64_t)r0 * (k / 32),
-                                                                                (const uint8_t*)w, (const uint8_t*)ws, yr, ob16, mm, n, k);
-                else fp8q_mfma_kernel<true><<<n / 16, 256, need(mm), st>>>((const uint16_t*)x + (int64_t)r0 * k, nullptr, nullptr, (const uint8_t*)w, (const uint8_t*)ws,
-                                                                           yr, ob16, mm, n, k);
+                const uint8_t* aqr = aq ? (const uint8_t*)aq + (int64_t)r0 * k : nullptr;
+                const uint8_t* asr = aq ? (const uint8_t*)as_ + (int64_t)r0 * (k / 32) : nullptr;
+                const uint16_t* xr = aq ? nullptr : (const uint16_t*)x + (int64_t)r0 * k;
+                if (aq && nw == 4) fp8q_mfma_kernel<false, 4><<<n / 16, 256, need(mm), st>>>(xr, aqr, asr, (const uint8_t*)w, (const uint8_t*)ws, yr, ob16, mm, n, k);
+                else if (aq) fp8q_mfma_kernel<false, 0><<<n / 16, 64 * nw, need(mm), st>>>(xr, aqr, asr, (const uint8_t*)w, (const uint8_t*)ws, yr, ob16, mm, n, k);
+                else if (nw == 4) fp8q_mfma_kernel<true, 4><<<n / 16, 256, need(mm), st>>>(xr, aqr, asr, (const uint8_t*)w, (const uint8_t*)ws, yr, ob16, mm, n, k);
+                else fp8q_mfma_kernel<true, 0><<<n / 16, 64 * nw, need(mm), st>>>(xr, aqr, asr, (const uint8_t*)w, (const uint8_t*)ws, yr, ob16, mm, n, k);
             }
             return launch_status();
         }

@@ -223,10 +223,12 @@ def test_fp8_gemv_bx_up_to_16_rows_and_groups(ops, oracle):
         assert rel_l2(yg[:, 64 * j:64 * j + 64], refj) < 1e-5
 
 
-@pytest.mark.parametrize("n,k,m", [(256, 1024, 11), (208, 2048, 21), (64, 4096, 3), (7168, 4096, 16)])
+@pytest.mark.parametrize("n,k,m", [(256, 1024, 11), (208, 2048, 21), (64, 4096, 3), (7168, 4096, 16), (160, 1280, 5), (128, 3072, 9), (1280, 5120, 3), (96, 768, 4),
+                                   (64, 1152, 4)])
 def test_fp8_gemv_with_quantised_activations(ops, oracle, n, k, m):
     # FP8 weights x act-quantised activations: every product is exact, the reference is the same sum in float64.  k a multiple of
-    # 2048 with n a multiple of 16 runs on the matrix unit (16 rows per launch), the first shape on the dot-product kernel
+    # 256 with n a multiple of 16 runs on the matrix unit (the reference model's 1280 / 3072 / 5120 among them), the last shape on
+    # the dot-product kernel
     g = synth.rng(151)
     w8, _ = synth.fp8_block_matrix(g, n, k)
     s8 = g.integers(110, 128, ((n + 31) // 32, k // 32), dtype=np.uint8)
