@@ -112,7 +112,7 @@ __global__ __launch_bounds__(DT) void dense_gemv_kernel(const void* __restrict__
 // The 4-bit case of the product above, the width every decode-time projection of the reference models has: the weight stream and
 // decode of the expert kernels.  grid (N / 128, S), 8 waves; a wave reads eight consecutive tiles of a k-tile row (1 KB) with one
 // 16-byte load per lane, four k-tiles in flight, decodes its 2 columns x 16 k per tile in registers and multiplies with
-// v_dot2_f32_f16 against the transformed rows in LDS; the waves' sums are added in wave order.  Up to 8 rows.
+// v_dot2_f32_f16 against the transformed rows in LDS; the waves' sums are added in wave order.  Up to 8 rows per launch.
 constexpr int D4_WAVES = 8, D4_FLY = 4;
 template <int CBK, int MR>
 __device__ __forceinline__ void tile_fma4(const uint4 w, uint32_t prev, const uint32_t* xrow, int ldx32, int rows, float (&acc)[MR][2])
@@ -127,8 +127,10 @@ __device__ __forceinline__ void tile_fma4(const uint4 w, uint32_t prev, const ui
 }
 template <int CBK, int MR, int XMODE>
 __global__ __launch_bounds__(64 * D4_WAVES) void dense4_gemv_kernel(const void* __restrict__ xin, int64_t ldx, const uint16_t* __restrict__ suh,
-                                                                    const uint32_t* __restrict__ tr, float* __restrict__ part, int M, int K, int N, int kts, int kpad)
+                                                                    const uint32_t* __restrict__ tr, float* __restrict__ part, int M, int K, int N, int kts, int kpad,
+                                                                    int Mtot, int r0)
 {
+    // M rows starting at row r0 of the call's Mtot (more than 8 rows run as passes of 8: the weights of a pass stream again)
     extern __shared__ __align__(16) unsigned char sm[];
     __shared__ float red[D4_WAVES][MR][128];
     const int Kt = K / 16, Nt = N / 16;
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(64 * D4_WAVES) void dense4_gemv_kernel(const void* 
     if (XMODE == 0) {
         for (int i = tid; i < M * (kpad / 2); i += 64 * D4_WAVES) {
             const int r = i / (kpad / 2), c = (i % (kpad / 2)) * 2;
-            *(uint32_t*)(xs + (size_t)r * kpad + c) = k0 + c < K ? *(const uint32_t*)((const uint16_t*)xin + (int64_t)r * K + k0 + c) : 0u;
+            *(uint32_t*)(xs + (size_t)r * kpad + c) = k0 + c < K ? *(const uint32_t*)((const uint16_t*)xin + (int64_t)(r0 + r) * K + k0 + c) : 0u;
         }
     } else {
         const int nblk = kpad / 128;
@@ -157,8 +159,8 @@ __global__ __launch_bounds__(64 * D4_WAVES) void dense4_gemv_kernel(const void* 
             const int r = u / nblk, k = k0 + (u % nblk) * 128 + 2 * lane;
             float v0 = 0.f, v1 = 0.f;
             if (k < K) {
-                v0 = ((const float*)xin)[r * ldx + k] * f16_bits_to_f32(suh[k]);
-                v1 = ((const float*)xin)[r * ldx + k + 1] * f16_bits_to_f32(suh[k + 1]);
+                v0 = ((const float*)xin)[(r0 + r) * ldx + k] * f16_bits_to_f32(suh[k]);
+                v1 = ((const float*)xin)[(r0 + r) * ldx + k + 1] * f16_bits_to_f32(suh[k + 1]);
             }
             fwht128(v0, v1, lane);
             *(uint32_t*)(xs + (size_t)r * kpad + (k - k0)) = (uint32_t)f32_to_f16_bits(v0) | ((uint32_t)f32_to_f16_bits(v1) << 16);
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(64 * D4_WAVES) void dense4_gemv_kernel(const void* 
         float v = red[0][r][c];
 #pragma unroll
         for (int w = 1; w < D4_WAVES; ++w) v += red[w][r][c];
-        part[((int64_t)s * M + r) * N + nb * 128 + c] = v;
+        part[((int64_t)s * Mtot + r0 + r) * N + nb * 128 + c] = v;
     }
 }
 
@@ -231,16 +233,19 @@ int launch_gemv(int xmode, const void* x, int64_t ldx, const void* suh, const vo
     const size_t smem = (size_t)M * kpad * 2 + 16 * 128 * 2 + 8 * 48 * 4;
     if (smem > 160 * 1024) return -1;
     const dim3 grid(N / 128, S);
-    if (bits == 4 && M <= 8) {
-        const size_t sm4 = (size_t)M * kpad * 2;
+    if (bits == 4) {
+        const size_t sm4 = (size_t)(M < 8 ? M : 8) * kpad * 2;
 #define D4(CB, MRR)                                                                                                                             \
     do {                                                                                                                                        \
-        if (xmode) dense4_gemv_kernel<CB, MRR, 1><<<grid, 64 * D4_WAVES, sm4, st>>>(x, ldx, (const uint16_t*)suh, (const uint32_t*)trellis, (float*)part, M, K, N, kts, kpad); \
-        else dense4_gemv_kernel<CB, MRR, 0><<<grid, 64 * D4_WAVES, sm4, st>>>(x, ldx, (const uint16_t*)suh, (const uint32_t*)trellis, (float*)part, M, K, N, kts, kpad);       \
+        if (xmode) dense4_gemv_kernel<CB, MRR, 1><<<grid, 64 * D4_WAVES, sm4, st>>>(x, ldx, (const uint16_t*)suh, (const uint32_t*)trellis, (float*)part, mm, K, N, kts, kpad, M, r0); \
+        else dense4_gemv_kernel<CB, MRR, 0><<<grid, 64 * D4_WAVES, sm4, st>>>(x, ldx, (const uint16_t*)suh, (const uint32_t*)trellis, (float*)part, mm, K, N, kts, kpad, M, r0);       \
     } while (0)
         if (sm4 <= 48 * 1024) {
-            if (codebook == CB_MCG) { if (M == 1) D4(CB_MCG, 1); else if (M == 2) D4(CB_MCG, 2); else if (M <= 4) D4(CB_MCG, 4); else D4(CB_MCG, 8); }
-            else { if (M == 1) D4(CB_MUL1, 1); else if (M == 2) D4(CB_MUL1, 2); else if (M <= 4) D4(CB_MUL1, 4); else D4(CB_MUL1, 8); }
+            for (int r0 = 0; r0 < M; r0 += 8) {
+                const int mm = M - r0 < 8 ? M - r0 : 8;
+                if (codebook == CB_MCG) { if (mm == 1) D4(CB_MCG, 1); else if (mm == 2) D4(CB_MCG, 2); else if (mm <= 4) D4(CB_MCG, 4); else D4(CB_MCG, 8); }
+                else { if (mm == 1) D4(CB_MUL1, 1); else if (mm == 2) D4(CB_MUL1, 2); else if (mm <= 4) D4(CB_MUL1, 4); else D4(CB_MUL1, 8); }
+            }
             return launch_status();
         }
 #undef D4

@@ -65,7 +65,7 @@ def test_linear_decode_shapes(ops, oracle):
     g = synth.rng(505)
     for K, N, S in ((2560, 512, 4), (640, 2560, 4), (640, 256, 3), (256, 128, 7)):
         tr, suh, svh = synth.exl3_matrix(g, K, N, 4)
-        for M in (1, 3, 8):
+        for M in (1, 3, 8, 21):
             x = g.standard_normal((M, K)).astype(np.float32)
             ref, _ = _reference(oracle, x, tr, suh, svh)
             y = host(ops.exl3_linear(dev(x), dev_f16(suh), dev(tr), dev_f16(svh), S=S))
