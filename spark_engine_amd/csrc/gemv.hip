@@ -766,34 +766,34 @@ int launch_qgemv(const void* x, const void* w, const void* sc, float* y, int m, 
             return launch_status();
         }
     }
-    if (m >= 3 && k % 512 == 0 && n % 16 == 0 && rpg == 0 && (FMT != 2 || bs == 128)) {     // three or more rows: the matrix unit
+    if (m >= 3 && k % 128 == 0 && n % 16 == 0 && rpg == 0 && (FMT != 2 || bs == 128)) {     // three or more rows: the matrix unit
         const size_t smm = (size_t)m * (k + MG_PAD) * 2;
-        if (smm <= MFMA_LDS_MAX) {
-            static bool attr = hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 4, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess &&
-                               hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 8, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess &&
-                               hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 4, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess &&
-                               hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 7, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess &&
-                               hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 8, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess;
+        // whole-line loads when a K part is whole chunks of 128 bytes a row: in eighths or sevenths for matrices whose row tiles
+        // leave a CU one workgroup, else in quarters, else in the parts K divides into (1280 -> fifths, 768 -> sixths or thirds)
+        const int cel = FMT == 0 ? 256 : 128;             // k per chunk
+        const size_t tile = (size_t)16 * MG_TS;
+        int kw = 0;
+        if (n / 16 <= 256 && k % (8 * cel) == 0) kw = 8;
+        else if (n / 16 <= 256 && k % (7 * cel) == 0) kw = 7;
+        else if (k % (4 * cel) == 0) kw = 4;
+        else for (int t : {5, 6, 3, 2, 1}) if (!kw && k % (t * cel) == 0) kw = t;
+        const size_t smt = ((smm + 15) & ~(size_t)15) + kw * tile;
+        if (kw && smt <= MFMA_LDS_MAX) {
+#define QM(KW)                                                                                                                                   \
+    do {                                                                                                                                         \
+        static bool attr = hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, KW, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess; \
+        if (!attr) return 3;                                                                                                                     \
+        q_mfma_gemv_kernel<FMT, KW, true><<<n / 16, 64 * KW, smt, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);             \
+    } while (0)
+            switch (kw) { case 8: QM(8); break; case 7: QM(7); break; case 6: QM(6); break; case 5: QM(5); break; case 4: QM(4); break; case 3: QM(3); break;
+                          case 2: QM(2); break; default: QM(1); }
+#undef QM
+            return launch_status();
+        }
+        if (k % 512 == 0 && smm <= MFMA_LDS_MAX) {          // operand-order loads (what no chunked split fits)
+            static bool attr = hipFuncSetAttribute((const void*)q_mfma_gemv_kernel<FMT, 4, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MFMA_LDS_MAX) == hipSuccess;
             if (!attr) return 3;
-            // whole-line loads when a K part is whole chunks of 128 bytes a row: in eighths or sevenths for matrices whose row tiles
-            // leave a CU one workgroup, else in quarters
-            {
-                const int cel = FMT == 0 ? 256 : 128;     // k per chunk
-                const size_t tile = (size_t)16 * MG_TS;
-                const int kw = n / 16 <= 256 && k % (8 * cel) == 0 ? 8 : n / 16 <= 256 && k % (7 * cel) == 0 ? 7 : k % (4 * cel) == 0 ? 4 : 0;
-                const size_t smt = ((smm + 15) & ~(size_t)15) + kw * tile;
-                if (kw && smt <= MFMA_LDS_MAX) {
-                    if (kw == 8) q_mfma_gemv_kernel<FMT, 8, true><<<n / 16, 512, smt, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
-                    else if (kw == 7) q_mfma_gemv_kernel<FMT, 7, true><<<n / 16, 448, smt, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
-                    else q_mfma_gemv_kernel<FMT, 4, true><<<n / 16, 256, smt, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
-                    return launch_status();
-                }
-            }
-            // K in quarters, or in eighths when the row tiles leave a CU with a single workgroup and an eighth is still six K blocks
-            // or more (4096 x 7168 at 4 rows: 13.5 -> 12.0 us; 7168 x 4096 in eighths: 11.9 -> 16.2 us).  The split depends on the
-            // shape only: a row's value does not depend on the row count
-            if (n / 16 <= 256 && k % 1024 == 0 && k >= 6144) q_mfma_gemv_kernel<FMT, 8, false><<<n / 16, 512, smm, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
-            else q_mfma_gemv_kernel<FMT, 4, false><<<n / 16, 256, smm, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
+            q_mfma_gemv_kernel<FMT, 4, false><<<n / 16, 256, smm, st>>>((const uint16_t*)x, xs, (const uint8_t*)w, sc, y, m, n, k);
             return launch_status();
         }
     }

@@ -164,7 +164,7 @@ def test_fp8_gemvs(ops, oracle, m):
     assert rel_l2(y, ref) < 1e-5
 
 
-@pytest.mark.parametrize("m,n,k", [(3, 208, 1536), (5, 64, 512), (8, 128, 4096), (4, 7168, 4096)])
+@pytest.mark.parametrize("m,n,k", [(3, 208, 1536), (5, 64, 512), (8, 128, 4096), (4, 7168, 4096), (6, 96, 1280), (8, 64, 768), (3, 48, 256)])
 def test_matrix_unit_gemvs(ops, oracle, m, n, k):
     # three or more rows of an eligible shape (k % 512 == 0, n % 16 == 0) run on the matrix unit in all three formats; the E8M0
     # scales span 50 binades inside a K block (they are applied relative to the block's largest)
