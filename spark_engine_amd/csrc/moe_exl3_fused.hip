@@ -8,9 +8,10 @@
 //       and up (Hadamard, svh), applies the activation and the down input transform and hands that block of xh2 to
 //       every down-projection block of the item.
 //   B blocks: (128-column block of H | item, K slice of 256).  Issue and DECODE their down-projection tiles first (they do not
-//       depend on stage 1), then take the item's xh2, dot; the last slice's block takes the other slices' sums and finishes
-//       (Hadamard, svh).  For every token row the block of
-//       the row's last item in launch order does the weighted slot-order sum for its 128 columns.
+//       depend on stage 1), then take the item's xh2, dot, and finish their own slice (the Hadamard transform is linear, so
+//       every slice is transformed on its own): Hadamard, svh, the pair's route weight.
+//   C blocks: (128-column block of H | token row).  They hold no weights: they wait for the topk * S2 finished slices of
+//       their row and add them in (slot, slice) order, four waves a share each, then the waves' sums in wave order.
 //
 // Exchange without counters: every exchanged 32-bit word of the workspace is EMPTY (all ones) between uses.  A producer
 // simply stores its value (a value that happens to be all ones, one particular NaN, is stored as another NaN); the one
@@ -20,16 +21,15 @@
 //
 // XCD-aware placement.  MI355X has 8 XCDs with one L2 each, and workgroup b runs on XCD b % 8 (checked once per process
 // by reading XCC_ID).  Block ids are laid out so that every exchange but one stays inside one XCD: the 2 * S1 blocks of
-// an (item, column block) group share an XCD, and so do all B blocks of one output column block (their experts' outputs
-// meet in the final sum).  Inside an XCD data moves through the shared L2 with ordinary stores and L1-bypassing loads.
+// an (item, column block) group share an XCD, and so do all B and C blocks of one output column block (their experts'
+// outputs meet in the final sum).  Inside an XCD data moves through the shared L2 with ordinary stores and L1-bypassing loads.
 // Only xh2 crosses XCDs, through device-coherent stores / loads.  If the placement check fails, every exchange uses the
 // device-coherent form.
 //
 // Order.  Every A block comes before every B block: a B block that waits for its item must not hold a slot an A block could
 // use (interleaving the two stages item by item was measured 17 % slower at one row and 46 % at four).
-// Progress.  Blocks are dispatched in id order and a block only ever waits for blocks with lower ids (A before B, the
-// finisher is the last block of its group, the summing block belongs to the row's last item), so whatever a block waits
-// for is resident or done.  Waits are bounded: on expiry the block sets an error flag and skips its work, and every
+// Progress.  Blocks are dispatched in id order and a block only ever waits for blocks with lower ids (A before B before C,
+// the finisher is the last block of its group), so whatever a block waits for is resident or done.  Waits are bounded: on expiry the block sets an error flag and skips its work, and every
 // block still runs to its end, so the grid always drains (the workspace must then be initialised again).
 //
 // Items are distinct experts in order of first appearance; rows of the per-pair buffers are the pair indices r * topk + k.
@@ -64,10 +64,9 @@ struct FArgs {
     const void* x; int64_t ldx; const void* idx; const void* w; const uint64_t* tab; const float* add; float* out;
     float* part1;                     // [S1][2][P][I] gate / up partial sums per K slice
     uint32_t* xh2;                    // [NB2][P][I / 2] packed fp16 pairs: one copy of the down input per consuming column block
-    float* part2;                     // [S2][P][H] down partial sums per K slice (S2 > 1 only)
-    float* yd;                        // [P][H] per-pair expert outputs
+    float* part2;                     // [S2][P][H] per pair and K slice of the down product: finished (Hadamard, svh) and weighted
     int* err;
-    int R, P, Gmax, S1, S2, NB1, NB2, nA, nB, bpgA, bpgB, local;     // S1 / S2 = K slices of stage 1 / 2
+    int R, P, Gmax, S1, S2, NB1, NB2, nA, nB, nC, bpgA, bpgB, local;     // S1 / S2 = K slices of stage 1 / 2
     Exl3Cfg c;
     long long* trace;                 // optional per-block timestamps (diagnostics), 8 per block
 };
@@ -162,18 +161,21 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
 {
     __shared__ __align__(16) uint16_t xs[MR][FW * TWMAX * 16];   // this block's K slice of the transformed activations (fp16)
     __shared__ float red[FW][MR][128];
-    __shared__ int sidx[PF_MAX], rows[RF_MAX], comb[RF_MAX], misc[4];
-    __shared__ float wsh[RF_MAX][16];                     // route weights of this item's token rows (stage 2)
+    __shared__ int sidx[PF_MAX], rows[RF_MAX], misc[4];
     __shared__ int owner[EMAX_F];                         // one int per expert id: scratch of the item lookup
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bid = blockIdx.x;
-    const bool isA = bid < a.nA;
+    const bool isA = bid < a.nA, isC = bid >= a.nA + a.nB;
     const Exl3Cfg& c = a.c;
     // ---- block id -> work.  Group q lives on XCD q % 8: bid = ((q / 8) * bpg + j) * 8 + q % 8, j = position in the group.
     int g = -1, t = 0, nb = 0, s = 0, K, N;
     {
-        const int b = isA ? bid : bid - a.nA, xcd = b % NXCD, li = b / NXCD;
-        if (isA) {
+        const int b = isA ? bid : isC ? bid - a.nA - a.nB : bid - a.nA, xcd = b % NXCD, li = b / NXCD;
+        if (isC) {
+            const int q = (li / a.R) * NXCD + xcd;                          // q = nb2, t = token row
+            if (q < a.NB2) { nb = q; t = li % a.R; s = 1; }                 // s = 1: this block has work
+            K = c.I; N = c.H;
+        } else if (isA) {
             const int j = li % a.bpgA, q = (li / a.bpgA) * NXCD + xcd;      // q = g * NB1 + nb1, j = t * S1 + s
             if (q < a.Gmax * a.NB1) { g = q / a.NB1; nb = q % a.NB1; t = j / a.S1; s = j % a.S1; }
             K = c.H; N = c.I;
@@ -196,7 +198,41 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
     Group grp{0, 0};
     if (g >= 0) grp = find_item(a, g, sidx, owner, rows, misc);
     TRACE(1);
-    if (grp.n > 0) {
+    if (isC) {
+        if (s) {
+            // ---- the row's topk * S2 finished slices, T words per lane pair, dealt to the waves in chunks of at most 8
+            const int ncol = nb * 128 + 2 * lane;
+            const int T = c.topk * a.S2, chunk = min(8, (T + FW - 1) / FW);
+            const float b0 = a.add ? a.add[(int64_t)t * c.H + ncol] : 0.f, b1 = a.add ? a.add[(int64_t)t * c.H + ncol + 1] : 0.f;
+            float a0 = 0.f, a1 = 0.f;
+            bool ok = true;
+            for (int q0 = wave * chunk; q0 < T; q0 += FW * chunk) {
+                const int n = min(chunk, T - q0);
+                float yl[8], yh[8];
+                float* py[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int q = q0 + (i < n ? i : 0);                     // slot q = (k, slice), k major
+                    py[i] = a.part2 + ((int64_t)(q % a.S2) * a.P + t * c.topk + q / a.S2) * c.H + ncol;
+                }
+                ok = take<LOCAL, 8>(py, n, yl, yh) && ok;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) if (i < n) { a0 += yl[i]; a1 += yh[i]; }
+            }
+            TRACE(4);
+            red[wave][0][2 * lane] = a0; red[wave][0][2 * lane + 1] = a1;
+            __syncthreads();
+            if (!ok && lane == 0) atomicExch(a.err, 1);
+            if (wave == 0 && ok) {
+                float v0 = red[0][0][2 * lane], v1 = red[0][0][2 * lane + 1];
+#pragma unroll
+                for (int w = 1; w < FW; ++w) { v0 += red[w][0][2 * lane]; v1 += red[w][0][2 * lane + 1]; }
+                a.out[(int64_t)t * c.H + ncol] = b0 + v0;
+                a.out[(int64_t)t * c.H + ncol + 1] = b1 + v1;
+            }
+            TRACE(6);
+        }
+    } else if (grp.n > 0) {
         const int Kt = K / 16, Nt = N / 16;
         const int ktb = FW * (isA ? TWA : TWB);           // k-tiles per block
         const int kt0 = s * ktb, kt1 = min(Kt, kt0 + ktb), nkt = kt1 - kt0;
@@ -329,26 +365,12 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
                 wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
             }
             TRACE(2);
-            const bool finisher = s == a.S2 - 1;
             const uint16_t* svd = (const uint16_t*)a.tab[(int64_t)8 * c.E + grp.e];
             const float svd0 = f16_bits_to_f32(svd[ncol]), svd1 = f16_bits_to_f32(svd[ncol + 1]);
-            // rows of this item whose weighted sum this block does: those whose other experts all belong to earlier items
-            if (finisher) {
-                for (int u = tid; u < grp.n * c.topk; u += 64 * FW)        // their route weights, fetched long before they are needed
-                    wsh[u / c.topk][u % c.topk] = exl3_ld_w(a.w, c.wtype, (rows[u / c.topk] / c.topk) * c.topk + u % c.topk);
-                if (a.R == 1) { if (tid == 0) comb[0] = g == a.P - 1; }
-                else {
-                    if (tid < grp.n) comb[tid] = 1;
-                    __syncthreads();
-                    const int fo = rows[0];               // first pair of this item's expert
-                    for (int u = tid; u < grp.n * c.topk; u += 64 * FW) {
-                        const int i = u / c.topk, k = u % c.topk, e = sidx[(rows[i] / c.topk) * c.topk + k];
-                        bool seen = false;
-                        for (int q = 0; q <= fo; ++q) seen |= sidx[q] == e;
-                        if (!seen) comb[i] = 0;
-                    }
-                }
-            }
+            // route weights of the pairs this wave finishes (rows wave, wave + FW, ...), fetched long before they are needed
+            float wk[(MR + FW - 1) / FW];
+#pragma unroll
+            for (int j = 0; j < (MR + FW - 1) / FW; ++j) wk[j] = exl3_ld_w(a.w, c.wtype, rows[wave + FW * j < grp.n ? wave + FW * j : 0]);
             h2 wd[TWB][4][4];
 #pragma unroll
             for (int i = 0; i < TWB; ++i) {
@@ -357,28 +379,45 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
                 for (int q = 0; q < 16; ++q) asm volatile("" : "+v"(wd[i][q >> 2][q & 3]));   // decoded now, not after the wait
             }
             asm volatile("" :: "v"(svd0), "v"(svd1));
+#pragma unroll
+            for (int j = 0; j < (MR + FW - 1) / FW; ++j) asm volatile("" :: "v"(wk[j]));
             TRACE(3);
             uint32_t* xc = a.xh2 + ((int64_t)nb * a.P) * (c.I / 2) + kt0 * 8;         // this column block's copy, this K slice
-            // cheap wait first: one word per 128-block of the slice (the finishers' last lanes), then every word
-            if (wave == 0) {
-                int spins = 0;
-                for (;;) {
-                    const uint32_t v = lane < nblk ? ld_dev32(xc + (int64_t)rows[0] * (c.I / 2) + lane * 64 + 63) : 0u;
-                    if (__builtin_amdgcn_ballot_w64(v == EMPTY) == 0 || ++spins >= SPIN_MAX) break;
-                    __builtin_amdgcn_s_sleep(4);
-                }
-            }
-            __syncthreads();
+            // One round per row: a wave watches whole rows of the slice (two words per lane, at most 128 words per row), so the
+            // data arrives with the poll that sees it complete; the other waves sleep at the barrier meanwhile.
             __builtin_amdgcn_s_setprio(3);                // from here on this block is the critical path
             bool good = true;
-            for (int u = tid; u < grp.n * (nkt * 8); u += 64 * FW) {                  // 2 fp16 per thread-step
-                const int r = u / (nkt * 8), q = u % (nkt * 8);
-                uint32_t* p = xc + (int64_t)rows[r] * (c.I / 2) + q;
-                uint32_t v;
-                int spins = 0;
-                while ((v = ld_dev32(p)) == EMPTY && ++spins < SPIN_MAX) __builtin_amdgcn_s_sleep(1);
-                if (v == EMPTY) good = false; else st_dev32(p, EMPTY);
-                *(uint32_t*)&xs[r][q * 2] = v;
+            {
+                constexpr int RW = (MR + FW - 1) / FW;    // rows per wave
+                uint32_t* p[RW];
+#pragma unroll
+                for (int j = 0; j < RW; ++j) {
+                    const int r = wave + FW * j;          // past the item's rows: this wave's first row again (never another wave's)
+                    p[j] = xc + (int64_t)rows[r < grp.n ? r : (wave < grp.n ? wave : 0)] * (c.I / 2) + (lane < nkt * 4 ? 2 * lane : 0);
+                }
+                if (wave < grp.n) {
+                    uint64_t v[RW];
+                    int spins = 0;
+                    for (;;) {
+                        asm volatile("" ::: "memory");
+                        bool ok = true;
+#pragma unroll
+                        for (int j = 0; j < RW; ++j) v[j] = ld_dev64(p[j]);
+#pragma unroll
+                        for (int j = 0; j < RW; ++j) ok = ok && (uint32_t)v[j] != EMPTY && (uint32_t)(v[j] >> 32) != EMPTY;
+                        if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+                        if (++spins >= SPIN_MAX) { good = false; break; }
+                        __builtin_amdgcn_s_sleep(2);
+                    }
+#pragma unroll
+                    for (int j = 0; j < RW; ++j) {
+                        const int r = wave + FW * j;
+                        if (r < grp.n && lane < nkt * 4) {
+                            if (good) st_dev64(p[j], EMPTY2);
+                            *(uint64_t*)&xs[r][4 * lane] = v[j];
+                        }
+                    }
+                }
             }
             if (!good) misc[2] = 0;
             __syncthreads();
@@ -399,68 +438,20 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
 #pragma unroll
                 for (int r = 0; r < MR; ++r) { red[wave][r][16 * j8 + m8] = acc[r][0]; red[wave][r][16 * j8 + m8 + 8] = acc[r][1]; }
                 __syncthreads();
-                if (!finisher) {
-                    float* part = a.part2 + ((int64_t)s * a.P) * N;
-                    for (int i = tid; i < grp.n * 64; i += 64 * FW) {
-                        const int r = i >> 6, col = (i & 63) * 2;
-                        float v0 = red[0][r][col], v1 = red[0][r][col + 1];
+                // ---- finish this slice of the down product (the transform is linear: slice by slice): Hadamard, svh, route
+                // weight; wave per pair row.  The C block of the token row adds the slices.
 #pragma unroll
-                        for (int w = 1; w < FW; ++w) { v0 += red[w][r][col]; v1 += red[w][r][col + 1]; }
-                        put2<LOCAL>(&part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
-                    }
-                    TRACE(6);
-                } else {
-                    // ---- finish the down product: yd[pair] = had128(sum of slices in order) * svh; wave per row
-                    bool ok = true;
-                    for (int r = wave; r < grp.n; r += FW) {
-                        float v0 = 0.f, v1 = 0.f;
-                        if (a.S2 == 2) {                   // the common split: one word pair, not a round of eight requests
-                            float pl[1], ph[1];
-                            float* pp[1] = {a.part2 + (int64_t)rows[r] * c.H + ncol};
-                            ok = take<LOCAL, 1>(pp, 1, pl, ph) && ok;
-                            v0 += pl[0]; v1 += ph[0];
-                        } else if (a.S2 > 2) {
-                            float pl[8], ph[8];
-                            float* pp[8];
-#pragma unroll
-                            for (int ss = 0; ss < 8; ++ss) pp[ss] = a.part2 + ((int64_t)(ss < a.S2 - 1 ? ss : 0) * a.P + rows[r]) * c.H + ncol;
-                            ok = take<LOCAL, 8>(pp, a.S2 - 1, pl, ph) && ok;
-#pragma unroll
-                            for (int ss = 0; ss < 8; ++ss) if (ss < a.S2 - 1) { v0 += pl[ss]; v1 += ph[ss]; }
-                        }
+                for (int j = 0; j < (MR + FW - 1) / FW; ++j) {
+                    const int r = wave + FW * j;
+                    if (r < grp.n) {
                         float o0 = red[0][r][2 * lane], o1 = red[0][r][2 * lane + 1];
 #pragma unroll
                         for (int w = 1; w < FW; ++w) { o0 += red[w][r][2 * lane]; o1 += red[w][r][2 * lane + 1]; }
-                        v0 += o0; v1 += o1;
-                        fwht128(v0, v1, lane);
-                        if (ok) put2<LOCAL>(a.yd + (int64_t)rows[r] * c.H + ncol, v0 * svd0, v1 * svd1);
+                        fwht128(o0, o1, lane);
+                        put2<LOCAL>(a.part2 + ((int64_t)s * a.P + rows[r]) * c.H + ncol, o0 * svd0 * wk[j], o1 * svd1 * wk[j]);
                     }
-                    TRACE(6);
-                    // ---- token rows this block sums: every expert's output of the row, in slot order, weighted
-                    for (int i = wave; i < grp.n; i += FW) {
-                        if (!comb[i]) continue;
-                        const int tr = rows[i] / c.topk;
-                        const float b0 = a.add ? a.add[(int64_t)tr * c.H + ncol] : 0.f, b1 = a.add ? a.add[(int64_t)tr * c.H + ncol + 1] : 0.f;
-                        float yl[16], yh[16];
-                        float* py[16];
-#pragma unroll
-                        for (int k = 0; k < 16; ++k) py[k] = a.yd + (int64_t)(tr * c.topk + (k < c.topk ? k : 0)) * c.H + ncol;
-                        ok = take<LOCAL, 16>(py, c.topk, yl, yh) && ok;
-                        TRACE(2);
-                        float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-                        for (int k = 0; k < 16; ++k)
-                            if (k < c.topk) {
-                                const float wk = wsh[i][k];
-                                a0 += wk * yl[k]; a1 += wk * yh[k];
-                            }
-                        if (ok) {
-                            a.out[(int64_t)tr * c.H + ncol] = b0 + a0;
-                            a.out[(int64_t)tr * c.H + ncol + 1] = b1 + a1;
-                        }
-                    }
-                    if (!ok && lane == 0) atomicExch(a.err, 1);
                 }
+                TRACE(6);
             } else if (tid == 0) atomicExch(a.err, 1);
         }
     }
@@ -480,7 +471,7 @@ __global__ void xcd_probe_kernel(int* out)
     if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((31 << 11) | 20) & 0xf;
 }
 
-struct FPlan { int P, Gmax, twa, S1, S2, NB1, NB2, nA, nB, bpgA, bpgB; size_t part1, xh2, part2, yd, total; };
+struct FPlan { int P, Gmax, twa, S1, S2, NB1, NB2, nA, nB, nC, bpgA, bpgB; size_t part1, xh2, part2, total; };
 FPlan fplan(const Exl3Cfg& c, int R)
 {
     FPlan p;
@@ -495,12 +486,12 @@ FPlan fplan(const Exl3Cfg& c, int R)
     const int QA = (p.Gmax * p.NB1 + NXCD - 1) / NXCD * NXCD, QB = (p.NB2 + NXCD - 1) / NXCD * NXCD;   // groups, padded to the XCD count
     p.nA = QA * p.bpgA;
     p.nB = QB * p.bpgB;
+    p.nC = QB * R;
     size_t o = HEAD;
     auto take = [&](size_t n) { const size_t q = o; o += align256(n); return q; };
     p.part1 = take(4 * (size_t)p.S1 * 2 * p.P * c.I);
     p.xh2 = take(4 * (size_t)p.NB2 * p.P * (c.I / 2));
-    p.part2 = take(p.S2 > 1 ? 4 * (size_t)p.S2 * p.P * c.H : 0);
-    p.yd = take(4 * (size_t)p.P * c.H);
+    p.part2 = take(4 * (size_t)p.S2 * p.P * c.H);
     p.total = o;
     return p;
 }
@@ -508,7 +499,7 @@ FPlan fplan(const Exl3Cfg& c, int R)
 template <int CBK, int TWA, bool LOCAL>
 void launch3(const FArgs& a, int maxrows, hipStream_t st)
 {
-    const dim3 grid(a.nA + a.nB), blk(64 * FW);
+    const dim3 grid(a.nA + a.nB + a.nC), blk(64 * FW);
     if (maxrows <= 1) fused_kernel<CBK, 1, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
     else if (maxrows <= 2) fused_kernel<CBK, 2, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
     else if (maxrows <= 4) fused_kernel<CBK, 4, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
@@ -565,8 +556,8 @@ int exl3_fused_launch(const Exl3Cfg& c, const void* x, int64_t ldx, int R, const
     char* b = (char*)ws;
     FArgs a;
     a.x = x; a.ldx = ldx; a.idx = idx; a.w = w; a.tab = (const uint64_t*)tab; a.add = (const float*)add; a.out = (float*)out;
-    a.err = (int*)b; a.part1 = (float*)(b + p.part1); a.xh2 = (uint32_t*)(b + p.xh2); a.part2 = (float*)(b + p.part2); a.yd = (float*)(b + p.yd);
-    a.R = R; a.P = p.P; a.Gmax = p.Gmax; a.S1 = p.S1; a.S2 = p.S2; a.NB1 = p.NB1; a.NB2 = p.NB2; a.nA = p.nA; a.nB = p.nB;
+    a.err = (int*)b; a.part1 = (float*)(b + p.part1); a.xh2 = (uint32_t*)(b + p.xh2); a.part2 = (float*)(b + p.part2);
+    a.R = R; a.P = p.P; a.Gmax = p.Gmax; a.S1 = p.S1; a.S2 = p.S2; a.NB1 = p.NB1; a.NB2 = p.NB2; a.nA = p.nA; a.nB = p.nB; a.nC = p.nC;
     a.bpgA = p.bpgA; a.bpgB = p.bpgB;
     a.local = g_xcd_local == 1;
     a.c = c;
