@@ -131,6 +131,15 @@ __device__ __forceinline__ void cvt_x2(int xtype, uint32_t r0, uint32_t r1, floa
     else { v0 = __uint_as_float(r0 << 16); v1 = __uint_as_float(r0 & 0xffff0000u); }
 }
 
+// A load whose address is the same for the whole wave, through the scalar cache: it does not queue behind the vector
+// loads (weight bursts) of the CU's other blocks, which cost a dependent lookup 1 - 2 us.  Only for memory the kernel
+// never writes (routing indices, route weights, the expert table).
+template <class T> __device__ __forceinline__ T ld_k(const T* p, int i)
+{
+    return *(const __attribute__((address_space(4))) T*)(uintptr_t)(p + __builtin_amdgcn_readfirstlane(i));
+}
+__device__ __forceinline__ int ld_idx_k(const void* idx, int itype, int i) { return itype ? (int)ld_k((const int64_t*)idx, i) : ld_k((const int*)idx, i); }
+
 struct Group { int e, n; };
 // item g of the call: expert and its pair rows (ascending) in rows[], or n = 0 when the call has fewer items.  All threads
 // call; wave 0 works the item out (one barrier).  Leaves every pair's expert in sidx[] when R > 1.
@@ -141,7 +150,7 @@ __device__ __forceinline__ Group find_item(const FArgs& a, int g, int* sidx, int
         if (g >= P) return Group{0, 0};
         if (tid == 0) rows[0] = g;
         __syncthreads();
-        return Group{exl3_ld_idx(a.idx, a.c.itype, g), 1};
+        return Group{ld_idx_k(a.idx, a.c.itype, g), 1};
     }
     if (tid < 64) {
         WaveItems<PF_MAX / 64> wi;
@@ -153,7 +162,7 @@ __device__ __forceinline__ Group find_item(const FArgs& a, int g, int* sidx, int
         if (tid == 0) { misc[0] = e; misc[1] = n; }
     }
     __syncthreads();
-    return misc[0] < 0 ? Group{0, 0} : Group{misc[0], misc[1]};
+    return misc[0] < 0 ? Group{0, 0} : Group{__builtin_amdgcn_readfirstlane(misc[0]), __builtin_amdgcn_readfirstlane(misc[1])};
 }
 
 template <int CBK, int MR, int TWA, bool LOCAL>
@@ -237,7 +246,7 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
         const int ktb = FW * (isA ? TWA : TWB);           // k-tiles per block
         const int kt0 = s * ktb, kt1 = min(Kt, kt0 + ktb), nkt = kt1 - kt0;
         const int nblk = (nkt + 7) / 8;                   // 128-blocks of K in this slice
-        const uint32_t* tr = (const uint32_t*)a.tab[(int64_t)(isA ? t : 2) * c.E + grp.e];
+        const uint32_t* tr = (const uint32_t*)ld_k(a.tab, (isA ? t : 2) * c.E + grp.e);
         const int src = tile_prev_lane(lane);
         const int ncol = nb * 128 + 2 * lane;             // this lane's two columns in the finishing steps
         const int j8 = lane >> 3, m8 = lane & 7;
@@ -247,7 +256,7 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
         if (isA) {
             const bool finisher = t == 1 && s == a.S1 - 1;
             // ---- the slice of x and its sign vector first (the transform overlaps the weight stream), then the tiles
-            const uint16_t* suh = (const uint16_t*)a.tab[(int64_t)(3 + t) * c.E + grp.e];
+            const uint16_t* suh = (const uint16_t*)ld_k(a.tab, (3 + t) * c.E + grp.e);
             uint32_t xr0, xr1, sr;
             const int unit0 = wave;                       // first (row, 128-block) unit of this wave
             {
@@ -268,9 +277,9 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
             // ---- scales of the finishing step (the finisher only)
             float sg0 = 0.f, sg1 = 0.f, su0 = 0.f, su1 = 0.f, sd0 = 0.f, sd1 = 0.f;
             if (finisher) {
-                const uint16_t* svg = (const uint16_t*)a.tab[(int64_t)6 * c.E + grp.e];
-                const uint16_t* svu = (const uint16_t*)a.tab[(int64_t)7 * c.E + grp.e];
-                const uint16_t* sud = (const uint16_t*)a.tab[(int64_t)5 * c.E + grp.e];
+                const uint16_t* svg = (const uint16_t*)ld_k(a.tab, 6 * c.E + grp.e);
+                const uint16_t* svu = (const uint16_t*)ld_k(a.tab, 7 * c.E + grp.e);
+                const uint16_t* sud = (const uint16_t*)ld_k(a.tab, 5 * c.E + grp.e);
                 sg0 = f16_bits_to_f32(svg[ncol]); sg1 = f16_bits_to_f32(svg[ncol + 1]);
                 su0 = f16_bits_to_f32(svu[ncol]); su1 = f16_bits_to_f32(svu[ncol + 1]);
                 sd0 = f16_bits_to_f32(sud[ncol]); sd1 = f16_bits_to_f32(sud[ncol + 1]);
@@ -319,6 +328,45 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
                     put2<LOCAL>(&part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
                 }
                 TRACE(6);
+            } else if (grp.n == 1) {
+                // ---- finisher of a one-row item, spread over the block (a lone wave's instruction chain is the cost here):
+                // wave 0 sums and transforms gate, wave 1 up; then every wave applies the activation and the down input
+                // transform itself and stores its share of the copies of xh2.  Same arithmetic as the general form below.
+                float* fin = (float*)&xs[0][0];           // [2][128]; the slice of x is no longer needed
+                const int r0 = rows[0];
+                if (wave < 2) {
+                    const int n = wave == 0 ? a.S1 : a.S1 - 1;             // this block holds the last up slice itself
+                    float pl[SMAX], ph[SMAX];
+                    float* pp[SMAX];
+#pragma unroll
+                    for (int ss = 0; ss < SMAX; ++ss) pp[ss] = a.part1 + ((int64_t)((ss < n ? ss : 0) * 2 + wave) * a.P + r0) * c.I + ncol;
+                    bool good = true;
+                    if (n > 0) good = take<LOCAL, SMAX>(pp, n, pl, ph);
+                    TRACE(4);
+                    float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+                    for (int ss = 0; ss < SMAX; ++ss) if (ss < n) { v0 += pl[ss]; v1 += ph[ss]; }
+                    if (wave == 1) {
+                        float o0 = red[0][0][2 * lane], o1 = red[0][0][2 * lane + 1];
+#pragma unroll
+                        for (int w = 1; w < FW; ++w) { o0 += red[w][0][2 * lane]; o1 += red[w][0][2 * lane + 1]; }
+                        v0 += o0; v1 += o1;
+                    }
+                    fwht128(v0, v1, lane);
+                    *(float2*)&fin[wave * 128 + 2 * lane] = make_float2(v0, v1);
+                    if (!good) misc[2] = 0;
+                }
+                __syncthreads();
+                if (misc[2]) {
+                    const float2 gg = *(const float2*)&fin[2 * lane], uu = *(const float2*)&fin[128 + 2 * lane];
+                    float v0 = exl3_act(c.act, gg.x * sg0, uu.x * su0) * sd0;
+                    float v1 = exl3_act(c.act, gg.y * sg1, uu.y * su1) * sd1;
+                    fwht128(v0, v1, lane);
+                    uint32_t pk = (uint32_t)f32_to_f16_bits(v0) | ((uint32_t)f32_to_f16_bits(v1) << 16);
+                    if (pk == EMPTY) pk = 0x7e007e00u;
+                    for (int q = wave; q < a.NB2; q += FW) st_dev32(a.xh2 + ((int64_t)q * a.P + r0) * (c.I / 2) + (ncol >> 1), pk);
+                } else if (tid == 0) atomicExch(a.err, 1);
+                TRACE(6);
             } else {
                 // ---- finisher: gate and up sums in slice order, Hadamard, svh, activation, down input transform -> xh2
                 bool good = true;
@@ -365,7 +413,7 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
                 wr[i] = ld_stream16(tr + ((int64_t)kt * Nt + nb * 8) * 32 + lane * 4);
             }
             TRACE(2);
-            const uint16_t* svd = (const uint16_t*)a.tab[(int64_t)8 * c.E + grp.e];
+            const uint16_t* svd = (const uint16_t*)ld_k(a.tab, 8 * c.E + grp.e);
             const float svd0 = f16_bits_to_f32(svd[ncol]), svd1 = f16_bits_to_f32(svd[ncol + 1]);
             // route weights of the pairs this wave finishes (rows wave, wave + FW, ...), fetched long before they are needed
             float wk[(MR + FW - 1) / FW];
