@@ -17,6 +17,14 @@ namespace spk {
 
 constexpr int WAVE = 64;
 
+// A load whose address is the same for the whole wave, through the scalar cache: it does not queue behind the vector
+// loads (weight bursts) of the CU's other blocks, which cost a dependent lookup 1 - 2 us.  Only for memory the kernel
+// never writes (routing indices, route weights, the expert table).
+template <class T> __device__ __forceinline__ T ld_k(const T* p, int i)
+{
+    return *(const __attribute__((address_space(4))) T*)(uintptr_t)(p + __builtin_amdgcn_readfirstlane(i));
+}
+
 // ---- number formats (bit-exact, software: the bytes must match the CPU reference of the same rule) ----
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
 __device__ __forceinline__ uint16_t f32_to_bf16(float f)

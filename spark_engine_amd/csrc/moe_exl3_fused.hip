@@ -131,13 +131,6 @@ __device__ __forceinline__ void cvt_x2(int xtype, uint32_t r0, uint32_t r1, floa
     else { v0 = __uint_as_float(r0 << 16); v1 = __uint_as_float(r0 & 0xffff0000u); }
 }
 
-// A load whose address is the same for the whole wave, through the scalar cache: it does not queue behind the vector
-// loads (weight bursts) of the CU's other blocks, which cost a dependent lookup 1 - 2 us.  Only for memory the kernel
-// never writes (routing indices, route weights, the expert table).
-template <class T> __device__ __forceinline__ T ld_k(const T* p, int i)
-{
-    return *(const __attribute__((address_space(4))) T*)(uintptr_t)(p + __builtin_amdgcn_readfirstlane(i));
-}
 __device__ __forceinline__ int ld_idx_k(const void* idx, int itype, int i) { return itype ? (int)ld_k((const int64_t*)idx, i) : ld_k((const int*)idx, i); }
 
 struct Group { int e, n; };

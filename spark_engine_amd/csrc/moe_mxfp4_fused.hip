@@ -75,6 +75,12 @@ __device__ __forceinline__ int pair_expert(const MArgs& a, int p)
     const int r = p / a.TT, k = p % a.TT;
     return k < a.topk ? (int)a.idx[(int64_t)r * a.topk + k] : a.E + (k - a.topk);
 }
+// the same for a pair index that is uniform over the wave: the index comes through the scalar cache
+__device__ __forceinline__ int pair_expert_k(const MArgs& a, int p)
+{
+    const int r = p / a.TT, k = p % a.TT;
+    return k < a.topk ? (int)ld_k(a.idx, r * a.topk + k) : a.E + (k - a.topk);
+}
 struct Group { int e, n; };      // an item: expert and number of pairs (rows), the pairs ascending in a rows[] array
 
 template <int LAYOUT, bool QUANT, bool LOCAL>
@@ -99,8 +105,8 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
     Group gu{0, 0}, gd{0, 0};
     const bool wantU = hasU, wantD = grpi >= 1 && bi < a.NBD;
     if (a.R == 1) {                                        // every pair is its own item
-        if (wantU && grpi < a.P) gu = Group{pair_expert(a, grpi), 1};
-        if (wantD && grpi - 1 < a.P) gd = Group{pair_expert(a, grpi - 1), 1};
+        if (wantU && grpi < a.P) gu = Group{pair_expert_k(a, grpi), 1};
+        if (wantD && grpi - 1 < a.P) gd = Group{pair_expert_k(a, grpi - 1), 1};
         if (tid == 0) { rowsU[0] = grpi; rowsD[0] = grpi - 1; }
         __syncthreads();
     } else {
