@@ -109,4 +109,30 @@ __device__ __forceinline__ void dot_tile32(const h2 (&wd)[4][4], const uint32_t*
     }
 }
 
+// The same products for four token rows at once on the matrix unit (v_mfma_f32_4x4x4_16b_f16: sixteen independent 4x4x4 blocks
+// of four lanes each).  As the B operand a lane supplies four consecutive k of one of its own columns, as the A operand the same
+// four k of token row lane % 4; the four values it gets back are rows 0..3 of that same column, so the results land where the
+// lane-wise dot products put them and the decode ALU does none of the multiplying.  xq[q] = activations k = 4q .. 4q+3 of
+// the lane's token row (fp16).  Rows are independent: a row's sum does not depend on what the other three hold.
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void mfma_tile32(const h2 (&wd)[4][4], const h4 (&xq)[4], v4f& a0, v4f& a1)
+{
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int j = 2 * (q & 1), c = q >> 1;             // k = 4q..4q+3 = pairs wd[j][c], wd[j+1][c] (column m), [c+2] (column m+8)
+        const h4 b0 = __builtin_shufflevector(wd[j][c], wd[j + 1][c], 0, 1, 2, 3);
+        const h4 b1 = __builtin_shufflevector(wd[j][c + 2], wd[j + 1][c + 2], 0, 1, 2, 3);
+        a0 = __builtin_amdgcn_mfma_f32_4x4x4f16(xq[q], b0, a0, 0, 0, 0);
+        a1 = __builtin_amdgcn_mfma_f32_4x4x4f16(xq[q], b1, a1, 0, 0, 0);
+    }
+}
+// the lane's A operands of one k-tile: 16 fp16 of its token row at xp (16-byte aligned)
+__device__ __forceinline__ void ld_xq(const uint16_t* xp, h4 (&xq)[4])
+{
+    const uint4 u0 = *(const uint4*)xp, u1 = *(const uint4*)(xp + 8);
+    const uint32_t w[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) { const uint2 t = make_uint2(w[2 * q], w[2 * q + 1]); __builtin_memcpy(&xq[q], &t, 8); }
+}
+
 }  // namespace spk

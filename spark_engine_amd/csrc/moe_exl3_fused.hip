@@ -243,9 +243,12 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
         const int src = tile_prev_lane(lane);
         const int ncol = nb * 128 + 2 * lane;             // this lane's two columns in the finishing steps
         const int j8 = lane >> 3, m8 = lane & 7;
-        float acc[MR][2];
+        // products on the matrix unit, four token rows per instruction: acc[h][c][i] = row 4h + i, column m8 (c = 0) or m8 + 8
+        constexpr int MH = (MR + 3) / 4;
+        v4f acc[MH][2];
 #pragma unroll
-        for (int r = 0; r < MR; ++r) { acc[r][0] = 0.f; acc[r][1] = 0.f; }
+        for (int h = 0; h < MH; ++h) { acc[h][0] = v4f{0.f, 0.f, 0.f, 0.f}; acc[h][1] = v4f{0.f, 0.f, 0.f, 0.f}; }
+        const int xrow = min(lane & 3, MR - 1);           // the token row whose activations this lane feeds (rows past the item's are ignored)
         if (isA) {
             const bool finisher = t == 1 && s == a.S1 - 1;
             // ---- the slice of x and its sign vector first (the transform overlaps the weight stream), then the tiles
@@ -300,16 +303,17 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
                     h2 wd[4][4];
                     decode_tile32<CBK>(wr[i], __shfl(wr[i].w, src, 64), wd);
 #pragma unroll
-                    for (int r = 0; r < MR; ++r) {
-                        if (r >= grp.n) break;
-                        dot_tile32(wd, (const uint32_t*)&xs[r][(kt - kt0) * 16], acc[r][0], acc[r][1]);
+                    for (int h = 0; h < MH; ++h) {
+                        h4 xq[4];
+                        ld_xq(&xs[min(4 * h + xrow, MR - 1)][(kt - kt0) * 16], xq);
+                        mfma_tile32(wd, xq, acc[h][0], acc[h][1]);
                     }
                 }
             }
             TRACE(5);
             // ---- sum the waves in wave order; every block but the finisher hands its partial over inside the XCD
 #pragma unroll
-            for (int r = 0; r < MR; ++r) { red[wave][r][16 * j8 + m8] = acc[r][0]; red[wave][r][16 * j8 + m8 + 8] = acc[r][1]; }
+            for (int r = 0; r < MR; ++r) { red[wave][r][16 * j8 + m8] = acc[r >> 2][0][r & 3]; red[wave][r][16 * j8 + m8 + 8] = acc[r >> 2][1][r & 3]; }
             __syncthreads();
             if (!finisher) {
                 float* part = a.part1 + ((int64_t)(s * 2 + t) * a.P) * N;
@@ -469,15 +473,16 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
                     const int kt = kt0 + wave + FW * i;
                     if (kt < kt1) {
 #pragma unroll
-                        for (int r = 0; r < MR; ++r) {
-                            if (r >= grp.n) break;
-                            dot_tile32(wd[i], (const uint32_t*)&xs[r][(kt - kt0) * 16], acc[r][0], acc[r][1]);
+                        for (int h = 0; h < MH; ++h) {
+                            h4 xq[4];
+                            ld_xq(&xs[min(4 * h + xrow, MR - 1)][(kt - kt0) * 16], xq);
+                            mfma_tile32(wd[i], xq, acc[h][0], acc[h][1]);
                         }
                     }
                 }
                 TRACE(5);
 #pragma unroll
-                for (int r = 0; r < MR; ++r) { red[wave][r][16 * j8 + m8] = acc[r][0]; red[wave][r][16 * j8 + m8 + 8] = acc[r][1]; }
+                for (int r = 0; r < MR; ++r) { red[wave][r][16 * j8 + m8] = acc[r >> 2][0][r & 3]; red[wave][r][16 * j8 + m8 + 8] = acc[r >> 2][1][r & 3]; }
                 __syncthreads();
                 // ---- finish this slice of the down product (the transform is linear: slice by slice): Hadamard, svh, route
                 // weight; wave per pair row.  The C block of the token row adds the slices.
@@ -512,6 +517,7 @@ __global__ void xcd_probe_kernel(int* out)
     if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((31 << 11) | 20) & 0xf;
 }
 
+int g_force_twa = 0;                  // diagnostics: 4 or 8 forces the k-tiles per wave of a stage-1 block, 0 = by shape
 struct FPlan { int P, Gmax, twa, S1, S2, NB1, NB2, nA, nB, nC, bpgA, bpgB; size_t part1, xh2, part2, total; };
 FPlan fplan(const Exl3Cfg& c, int R)
 {
@@ -520,6 +526,7 @@ FPlan fplan(const Exl3Cfg& c, int R)
     p.Gmax = p.P < c.E ? p.P : c.E;
     // finer stage-1 blocks balance the CUs better while the grid is small (and K allows 8 slices)
     p.twa = c.H / 16 <= SMAX * FW * 4 && (int64_t)p.Gmax * (c.I / 128) * 2 * (c.H / 16 / (FW * 4)) <= 1024 ? 4 : 8;
+    if (g_force_twa == 8 || (g_force_twa == 4 && c.H / 16 <= SMAX * FW * 4)) p.twa = g_force_twa;
     p.S1 = (c.H / 16 + FW * p.twa - 1) / (FW * p.twa);
     p.S2 = (c.I / 16 + FW * TWB - 1) / (FW * TWB);
     p.NB1 = c.I / 128; p.NB2 = c.H / 128;
@@ -614,6 +621,8 @@ int exl3_fused_launch(const Exl3Cfg& c, const void* x, int64_t ldx, int R, const
 
 // diagnostics: device buffer of 8 timestamps (100 MHz) per block of the next launches, or null
 extern "C" __attribute__((visibility("default"))) void spark_debug_exl3_trace(long long* buf) { g_trace = buf; }
+// diagnostics: force the k-tiles per wave of a stage-1 block (4 or 8; 0 = chosen by shape)
+extern "C" __attribute__((visibility("default"))) void spark_debug_exl3_twa(int v) { g_force_twa = v; }
 // diagnostics: force the exchange mode of the single-launch path (1 XCD-local, 0 device-coherent, -1 probe again)
 extern "C" __attribute__((visibility("default"))) void spark_debug_exl3_local(int v) { g_xcd_local = v; }
 
