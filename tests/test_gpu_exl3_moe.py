@@ -29,7 +29,10 @@ def _to_dev(experts):
 
 
 @pytest.mark.parametrize("cbk,act", [(2, 0), (1, 1)])
-@pytest.mark.parametrize("R,H,I,E,topk", [(1, 256, 128, 4, 2), (1, 2048, 512, 512, 10), (4, 2048, 512, 512, 10), (3, 512, 384, 16, 4)])
+# the last two: twelve slots x four K slices of the down product (the summing blocks take their slices in two rounds), and
+# eight rows over eight experts with a ragged last K slice (items of several rows, two rows per wave in the stage-2 wait)
+@pytest.mark.parametrize("R,H,I,E,topk", [(1, 256, 128, 4, 2), (1, 2048, 512, 512, 10), (4, 2048, 512, 512, 10), (3, 512, 384, 16, 4),
+                                          (3, 512, 1024, 32, 12), (8, 256, 640, 8, 3)])
 def test_exl3_moe_vs_oracle(ops, oracle, cbk, act, R, H, I, E, topk):
     g = synth.rng(400 + R + H + cbk)
     logits = g.standard_normal((R, E)).astype(np.float32)
