@@ -353,7 +353,7 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
             for (;;) {
                 const uint32_t v = lane < nblk ? ld_dev32(a.hsw + ((int64_t)nb * a.P + rows[0]) * (I >> 5) + kg * 16 + lane) : 0u;
                 if (__builtin_amdgcn_ballot_w64(v == EMPTY) == 0 || ++spins >= SPIN_MAX) break;
-                __builtin_amdgcn_s_sleep(4);
+                __builtin_amdgcn_s_sleep(16);
             }
             if (valid) {
                 const int64_t row = (int64_t)nb * a.P + rows[c];
