@@ -524,8 +524,10 @@ FPlan fplan(const Exl3Cfg& c, int R)
     FPlan p;
     p.P = R * c.topk;
     p.Gmax = p.P < c.E ? p.P : c.E;
-    // finer stage-1 blocks balance the CUs better while the grid is small (and K allows 8 slices)
-    p.twa = c.H / 16 <= SMAX * FW * 4 && (int64_t)p.Gmax * (c.I / 128) * 2 * (c.H / 16 / (FW * 4)) <= 1024 ? 4 : 8;
+    // The K slices (and with them the order of summation) depend on the shape only, never on R: a row's bits must not depend on
+    // the batch.  Four k-tiles per wave wherever K allows 8 slices: finer stage-1 blocks balance the CUs better at one and two
+    // rows (the common decode calls); eight would be 5 % faster at four rows and 8 % at eight.
+    p.twa = c.H / 16 <= SMAX * FW * 4 ? 4 : 8;
     if (g_force_twa == 8 || (g_force_twa == 4 && c.H / 16 <= SMAX * FW * 4)) p.twa = g_force_twa;
     p.S1 = (c.H / 16 + FW * p.twa - 1) / (FW * p.twa);
     p.S2 = (c.I / 16 + FW * TWB - 1) / (FW * TWB);

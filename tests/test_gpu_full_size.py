@@ -85,3 +85,28 @@ def test_c5_prefill_rows_equal_decode_rows(ops, oracle):
         sub = [host(a[used]) for a in t]
         ref = oracle.mxfp4_moe(x[r:r + 1], np.array([[remap[e] for e in idx[r]]], np.int64), rw[r:r + 1], *sub)
         assert rel_l2(yh[r:r + 1], ref) <= TOL
+
+
+def test_c2_layer_rows_do_not_depend_on_the_batch(ops, oracle):
+    # hidden 2048, intermediate 512, 512 experts top-10 (the table holds the experts the routes use): a token row gives the
+    # same bits alone, in a call of four rows and in a call of eight (reference engine-rs/src/ds41/kern.rs:1886-1907,
+    # qwen_tests/test_kern_moe.py:23-24), and matches the oracle
+    H, I, E, topk, R = 2048, 512, 512, 10, 8
+    g = synth.rng(630)
+    logits = g.standard_normal((R, E)).astype(np.float32)
+    idx, w = oracle.qwen_route(logits, topk)
+    used = sorted(set(idx.ravel().tolist()))
+    experts = {e: synth.exl3_expert(g, H, I) for e in used}
+    from spark_engine_amd.ops import ExpertTable
+    from tests.gpu_util import dev_f16
+    table = ExpertTable({e: [dev(t[0]), dev(t[1]), dev(t[2])] + [dev_f16(a) for a in t[3:]] for e, t in experts.items()}, E)
+    xb = synth.randn_bf16(g, (R, H))
+    xd, idxd, wd = dev_bf16(xb), dev(idx), dev(w)
+    y8 = host(ops.exl3_moe(xd, idxd, wd, table, H, I))
+    ref = oracle.exl3_moe(synth.bf16_to_f32(xb), idx, w, experts, E, H, I, 4, 2, 0)
+    assert rel_l2(y8, ref) <= TOL, rel_l2(y8, ref)
+    y4 = host(ops.exl3_moe(xd[:4], idxd[:4], wd[:4], table, H, I))
+    assert np.array_equal(y4, y8[:4])
+    for r in (0, 3, 7):
+        y1 = host(ops.exl3_moe(xd[r:r + 1], idxd[r:r + 1], wd[r:r + 1], table, H, I))
+        assert np.array_equal(y1[0], y8[r]), r
