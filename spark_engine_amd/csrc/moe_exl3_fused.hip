@@ -66,7 +66,7 @@ struct FArgs {
     uint32_t* xh2;                    // [NB2][P][I / 2] packed fp16 pairs: one copy of the down input per consuming column block
     float* part2;                     // [S2][P][H] per pair and K slice of the down product: finished (Hadamard, svh) and weighted
     int* err;
-    int R, P, Gmax, S1, S2, NB1, NB2, nA, nB, nC, bpgA, bpgB, local;     // S1 / S2 = K slices of stage 1 / 2
+    int R, P, Gmax, S1, VS, S2, NB1, NB2, nA, nB, nC, bpgA, bpgB, local;     // S1 / S2 = blocks along K of stage 1 / 2; VS = K slices of stage 1 (NH per block)
     Exl3Cfg c;
     long long* trace;                 // optional per-block timestamps (diagnostics), 8 per block
 };
@@ -158,7 +158,7 @@ __device__ __forceinline__ Group find_item(const FArgs& a, int g, int* sidx, int
     return misc[0] < 0 ? Group{0, 0} : Group{__builtin_amdgcn_readfirstlane(misc[0]), __builtin_amdgcn_readfirstlane(misc[1])};
 }
 
-template <int CBK, int MR, int TWA, bool LOCAL>
+template <int CBK, int MR, int TWA, int NH, bool LOCAL>
 __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
 {
     __shared__ __align__(16) uint16_t xs[MR][FW * TWMAX * 16];   // this block's K slice of the transformed activations (fp16)
@@ -296,6 +296,11 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
             }
             __syncthreads();
             TRACE(3);
+            // A block of eight k-tiles per wave keeps one sum per half (NH = 2): a K slice is always sixteen k-tiles summed in the
+            // same order, whatever the block size, so a row's bits do not depend on the block size a call's grid asks for.
+            v4f acc2[NH == 2 ? MH : 1][2];
+#pragma unroll
+            for (int h = 0; h < (NH == 2 ? MH : 1); ++h) { acc2[h][0] = v4f{0.f, 0.f, 0.f, 0.f}; acc2[h][1] = v4f{0.f, 0.f, 0.f, 0.f}; }
 #pragma unroll
             for (int i = 0; i < TWA; ++i) {
                 const int kt = kt0 + wave + FW * i;
@@ -306,33 +311,48 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
                     for (int h = 0; h < MH; ++h) {
                         h4 xq[4];
                         ld_xq(&xs[min(4 * h + xrow, MR - 1)][(kt - kt0) * 16], xq);
-                        mfma_tile32(wd, xq, acc[h][0], acc[h][1]);
+                        if (NH == 2 && i >= 4) mfma_tile32(wd, xq, acc2[h][0], acc2[h][1]);
+                        else mfma_tile32(wd, xq, acc[h][0], acc[h][1]);
                     }
                 }
             }
             TRACE(5);
-            // ---- sum the waves in wave order; every block but the finisher hands its partial over inside the XCD
+            // ---- per K slice: sum the waves in wave order; every block but the finisher hands the slice over inside the XCD, the
+            // finisher keeps its own slices in LDS (where the activations were: every wave is past them after the first barrier)
+            float* ownl = (float*)&xs[0][0];              // [NH][MR][128]
+            const int nh = NH == 1 ? 1 : min(NH, (nkt + 15) / 16);          // K slices of this block that hold k-tiles
 #pragma unroll
-            for (int r = 0; r < MR; ++r) { red[wave][r][16 * j8 + m8] = acc[r >> 2][0][r & 3]; red[wave][r][16 * j8 + m8 + 8] = acc[r >> 2][1][r & 3]; }
-            __syncthreads();
-            if (!finisher) {
-                float* part = a.part1 + ((int64_t)(s * 2 + t) * a.P) * N;
-                for (int i = tid; i < grp.n * 64; i += 64 * FW) {
-                    const int r = i >> 6, col = (i & 63) * 2;
-                    float v0 = red[0][r][col], v1 = red[0][r][col + 1];
+            for (int hf = 0; hf < NH; ++hf) {
+                if (hf < nh) {
+                    if (hf) __syncthreads();              // the previous slice's sums have been read
 #pragma unroll
-                    for (int w = 1; w < FW; ++w) { v0 += red[w][r][col]; v1 += red[w][r][col + 1]; }
-                    put2<LOCAL>(&part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
+                    for (int r = 0; r < MR; ++r) {
+                        red[wave][r][16 * j8 + m8] = (NH == 2 && hf ? acc2 : acc)[r >> 2][0][r & 3];
+                        red[wave][r][16 * j8 + m8 + 8] = (NH == 2 && hf ? acc2 : acc)[r >> 2][1][r & 3];
+                    }
+                    __syncthreads();
+                    float* part = a.part1 + ((int64_t)((s * NH + hf) * 2 + t) * a.P) * N;
+                    for (int i = tid; i < grp.n * 64; i += 64 * FW) {
+                        const int r = i >> 6, col = (i & 63) * 2;
+                        float v0 = red[0][r][col], v1 = red[0][r][col + 1];
+#pragma unroll
+                        for (int w = 1; w < FW; ++w) { v0 += red[w][r][col]; v1 += red[w][r][col + 1]; }
+                        if (!finisher) put2<LOCAL>(&part[(int64_t)rows[r] * N + nb * 128 + col], v0, v1);
+                        else { ownl[(hf * MR + r) * 128 + col] = v0; ownl[(hf * MR + r) * 128 + col + 1] = v1; }
+                    }
                 }
+            }
+            if (!finisher) {
                 TRACE(6);
             } else if (grp.n == 1) {
+                __syncthreads();                          // the own slices are in place and the waves' sums are free
                 // ---- finisher of a one-row item, spread over the block (a lone wave's instruction chain is the cost here):
                 // wave 0 sums and transforms gate, wave 1 up; then every wave applies the activation and the down input
                 // transform itself and stores its share of the copies of xh2.  Same arithmetic as the general form below.
-                float* fin = (float*)&xs[0][0];           // [2][128]; the slice of x is no longer needed
+                float* fin = &red[0][0][0];               // [2][128]
                 const int r0 = rows[0];
                 if (wave < 2) {
-                    const int n = wave == 0 ? a.S1 : a.S1 - 1;             // this block holds the last up slice itself
+                    const int n = wave == 0 ? a.VS : a.VS - nh;            // this block holds the last up slices itself
                     float pl[SMAX], ph[SMAX];
                     float* pp[SMAX];
 #pragma unroll
@@ -344,10 +364,8 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
 #pragma unroll
                     for (int ss = 0; ss < SMAX; ++ss) if (ss < n) { v0 += pl[ss]; v1 += ph[ss]; }
                     if (wave == 1) {
-                        float o0 = red[0][0][2 * lane], o1 = red[0][0][2 * lane + 1];
 #pragma unroll
-                        for (int w = 1; w < FW; ++w) { o0 += red[w][0][2 * lane]; o1 += red[w][0][2 * lane + 1]; }
-                        v0 += o0; v1 += o1;
+                        for (int hf = 0; hf < NH; ++hf) if (hf < nh) { v0 += ownl[hf * MR * 128 + 2 * lane]; v1 += ownl[hf * MR * 128 + 2 * lane + 1]; }
                     }
                     fwht128(v0, v1, lane);
                     *(float2*)&fin[wave * 128 + 2 * lane] = make_float2(v0, v1);
@@ -366,28 +384,28 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
                 TRACE(6);
             } else {
                 // ---- finisher: gate and up sums in slice order, Hadamard, svh, activation, down input transform -> xh2
+                __syncthreads();                          // the own slices are in place
                 bool good = true;
                 for (int r = wave; r < grp.n; r += FW) {
-                    // gate slices 0 .. S1-1 and up slices 0 .. S1-2 (this block holds the last up slice itself), one round of requests
+                    // gate slices 0 .. VS-1 and up slices 0 .. VS-nh-1 (this block holds the last up slices itself), one round of requests
                     float pl[2 * SMAX], ph[2 * SMAX];
                     float* pp[2 * SMAX];
 #pragma unroll
                     for (int ss = 0; ss < 2 * SMAX; ++ss) {
-                        const int tt = ss < a.S1 ? 0 : 1, s2 = ss < a.S1 ? ss : (ss - a.S1 < a.S1 - 1 ? ss - a.S1 : 0);
+                        const int tt = ss < a.VS ? 0 : 1, s2 = ss < a.VS ? ss : (ss - a.VS < a.VS - nh ? ss - a.VS : 0);
                         pp[ss] = a.part1 + ((int64_t)(s2 * 2 + tt) * a.P + rows[r]) * c.I + ncol;
                     }
-                    good = take<LOCAL, 2 * SMAX>(pp, 2 * a.S1 - 1, pl, ph) && good;
+                    good = take<LOCAL, 2 * SMAX>(pp, 2 * a.VS - nh, pl, ph) && good;
                     TRACE(4);
                     float g0 = 0.f, g1 = 0.f, u0 = 0.f, u1 = 0.f;
 #pragma unroll
                     for (int ss = 0; ss < 2 * SMAX; ++ss) {
-                        if (ss < a.S1) { g0 += pl[ss]; g1 += ph[ss]; }
-                        else if (ss < 2 * a.S1 - 1) { u0 += pl[ss]; u1 += ph[ss]; }
+                        if (ss < a.VS) { g0 += pl[ss]; g1 += ph[ss]; }
+                        else if (ss < 2 * a.VS - nh) { u0 += pl[ss]; u1 += ph[ss]; }
                     }
-                    float o0 = red[0][r][2 * lane], o1 = red[0][r][2 * lane + 1];      // this block's own slice of up, last in order
 #pragma unroll
-                    for (int w = 1; w < FW; ++w) { o0 += red[w][r][2 * lane]; o1 += red[w][r][2 * lane + 1]; }
-                    u0 += o0; u1 += o1;
+                    for (int hf = 0; hf < NH; ++hf)           // this block's own slices of up, last in order
+                        if (hf < nh) { u0 += ownl[(hf * MR + r) * 128 + 2 * lane]; u1 += ownl[(hf * MR + r) * 128 + 2 * lane + 1]; }
                     fwht128(g0, g1, lane);
                     fwht128(u0, u1, lane);
                     float v0 = exl3_act(c.act, g0 * sg0, u0 * su0) * sd0;
@@ -518,18 +536,21 @@ __global__ void xcd_probe_kernel(int* out)
 }
 
 int g_force_twa = 0;                  // diagnostics: 4 or 8 forces the k-tiles per wave of a stage-1 block, 0 = by shape
-struct FPlan { int P, Gmax, twa, S1, S2, NB1, NB2, nA, nB, nC, bpgA, bpgB; size_t part1, xh2, part2, total; };
+struct FPlan { int P, Gmax, twa, nh, S1, VS, S2, NB1, NB2, nA, nB, nC, bpgA, bpgB; size_t part1, xh2, part2, total; };
 FPlan fplan(const Exl3Cfg& c, int R)
 {
     FPlan p;
     p.P = R * c.topk;
     p.Gmax = p.P < c.E ? p.P : c.E;
     // The K slices (and with them the order of summation) depend on the shape only, never on R: a row's bits must not depend on
-    // the batch.  Four k-tiles per wave wherever K allows 8 slices: finer stage-1 blocks balance the CUs better at one and two
-    // rows (the common decode calls); eight would be 5 % faster at four rows and 8 % at eight.
-    p.twa = c.H / 16 <= SMAX * FW * 4 ? 4 : 8;
-    if (g_force_twa == 8 || (g_force_twa == 4 && c.H / 16 <= SMAX * FW * 4)) p.twa = g_force_twa;
+    // the batch.  Where K allows 8 slices of sixteen k-tiles, a slice is sixteen k-tiles; finer stage-1 blocks (one slice each)
+    // balance the CUs better while the grid is small, larger blocks (two slices each, summed apart) turn over less when it is not.
+    const bool fine = c.H / 16 <= SMAX * FW * 4;
+    p.twa = fine && (int64_t)p.Gmax * (c.I / 128) * 2 * (c.H / 16 / (FW * 4)) <= 1536 ? 4 : 8;   // measured: C2 at two rows (1280 blocks) is faster fine, at four (2560) coarse
+    if (g_force_twa == 8 || (g_force_twa == 4 && fine)) p.twa = g_force_twa;
+    p.nh = p.twa == 8 && fine ? 2 : 1;
     p.S1 = (c.H / 16 + FW * p.twa - 1) / (FW * p.twa);
+    p.VS = p.nh == 2 ? (c.H / 16 + FW * 4 - 1) / (FW * 4) : p.S1;
     p.S2 = (c.I / 16 + FW * TWB - 1) / (FW * TWB);
     p.NB1 = c.I / 128; p.NB2 = c.H / 128;
     p.bpgA = 2 * p.S1; p.bpgB = p.Gmax * p.S2;
@@ -539,27 +560,33 @@ FPlan fplan(const Exl3Cfg& c, int R)
     p.nC = QB * R;
     size_t o = HEAD;
     auto take = [&](size_t n) { const size_t q = o; o += align256(n); return q; };
-    p.part1 = take(4 * (size_t)p.S1 * 2 * p.P * c.I);
+    p.part1 = take(4 * (size_t)p.VS * 2 * p.P * c.I);
     p.xh2 = take(4 * (size_t)p.NB2 * p.P * (c.I / 2));
     p.part2 = take(4 * (size_t)p.S2 * p.P * c.H);
     p.total = o;
     return p;
 }
 
-template <int CBK, int TWA, bool LOCAL>
+template <int CBK, int TWA, int NH, bool LOCAL>
 void launch3(const FArgs& a, int maxrows, hipStream_t st)
 {
     const dim3 grid(a.nA + a.nB + a.nC), blk(64 * FW);
-    if (maxrows <= 1) fused_kernel<CBK, 1, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
-    else if (maxrows <= 2) fused_kernel<CBK, 2, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
-    else if (maxrows <= 4) fused_kernel<CBK, 4, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
-    else fused_kernel<CBK, 8, TWA, LOCAL><<<grid, blk, 0, st>>>(a);
+    if (maxrows <= 1) fused_kernel<CBK, 1, TWA, NH, LOCAL><<<grid, blk, 0, st>>>(a);
+    else if (maxrows <= 2) fused_kernel<CBK, 2, TWA, NH, LOCAL><<<grid, blk, 0, st>>>(a);
+    else if (maxrows <= 4) fused_kernel<CBK, 4, TWA, NH, LOCAL><<<grid, blk, 0, st>>>(a);
+    else fused_kernel<CBK, 8, TWA, NH, LOCAL><<<grid, blk, 0, st>>>(a);
+}
+template <int CBK, bool LOCAL>
+void launch2(const FArgs& a, int twa, int nh, int maxrows, hipStream_t st)
+{
+    if (twa == 4) launch3<CBK, 4, 1, LOCAL>(a, maxrows, st);
+    else if (nh == 2) launch3<CBK, 8, 2, LOCAL>(a, maxrows, st);
+    else launch3<CBK, 8, 1, LOCAL>(a, maxrows, st);
 }
 template <int CBK>
-void launch(const FArgs& a, int twa, int maxrows, hipStream_t st)
+void launch(const FArgs& a, int twa, int nh, int maxrows, hipStream_t st)
 {
-    if (a.local) { if (twa == 4) launch3<CBK, 4, true>(a, maxrows, st); else launch3<CBK, 8, true>(a, maxrows, st); }
-    else { if (twa == 4) launch3<CBK, 4, false>(a, maxrows, st); else launch3<CBK, 8, false>(a, maxrows, st); }
+    if (a.local) launch2<CBK, true>(a, twa, nh, maxrows, st); else launch2<CBK, false>(a, twa, nh, maxrows, st);
 }
 
 int g_xcd_local = -1;                 // -1 unknown, 0 placement check failed, 1 workgroup b runs on XCD b % 8
@@ -607,7 +634,7 @@ int exl3_fused_launch(const Exl3Cfg& c, const void* x, int64_t ldx, int R, const
     FArgs a;
     a.x = x; a.ldx = ldx; a.idx = idx; a.w = w; a.tab = (const uint64_t*)tab; a.add = (const float*)add; a.out = (float*)out;
     a.err = (int*)b; a.part1 = (float*)(b + p.part1); a.xh2 = (uint32_t*)(b + p.xh2); a.part2 = (float*)(b + p.part2);
-    a.R = R; a.P = p.P; a.Gmax = p.Gmax; a.S1 = p.S1; a.S2 = p.S2; a.NB1 = p.NB1; a.NB2 = p.NB2; a.nA = p.nA; a.nB = p.nB; a.nC = p.nC;
+    a.R = R; a.P = p.P; a.Gmax = p.Gmax; a.S1 = p.S1; a.VS = p.VS; a.S2 = p.S2; a.NB1 = p.NB1; a.NB2 = p.NB2; a.nA = p.nA; a.nB = p.nB; a.nC = p.nC;
     a.bpgA = p.bpgA; a.bpgB = p.bpgB;
     a.local = g_xcd_local == 1;
     a.c = c;
@@ -616,8 +643,8 @@ int exl3_fused_launch(const Exl3Cfg& c, const void* x, int64_t ldx, int R, const
         const int rc = exl3_fused_ws_prepare(ws, p.total, st);
         if (rc) return rc;
     }
-    if (c.cbk == CB_MCG) launch<CB_MCG>(a, p.twa, R, st);
-    else launch<CB_MUL1>(a, p.twa, R, st);
+    if (c.cbk == CB_MCG) launch<CB_MCG>(a, p.twa, p.nh, R, st);
+    else launch<CB_MUL1>(a, p.twa, p.nh, R, st);
     return launch_status();
 }
 

@@ -105,8 +105,9 @@ def test_c2_layer_rows_do_not_depend_on_the_batch(ops, oracle):
     y8 = host(ops.exl3_moe(xd, idxd, wd, table, H, I))
     ref = oracle.exl3_moe(synth.bf16_to_f32(xb), idx, w, experts, E, H, I, 4, 2, 0)
     assert rel_l2(y8, ref) <= TOL, rel_l2(y8, ref)
-    y4 = host(ops.exl3_moe(xd[:4], idxd[:4], wd[:4], table, H, I))
-    assert np.array_equal(y4, y8[:4])
+    for n in (4, 2):                                                    # calls of two rows run smaller stage-1 blocks than calls of four
+        yn = host(ops.exl3_moe(xd[:n], idxd[:n], wd[:n], table, H, I))
+        assert np.array_equal(yn, y8[:n]), n
     for r in (0, 3, 7):
         y1 = host(ops.exl3_moe(xd[r:r + 1], idxd[r:r + 1], wd[r:r + 1], table, H, I))
         assert np.array_equal(y1[0], y8[r]), r
