@@ -43,14 +43,27 @@ __device__ __forceinline__ uint32_t fkey(float f)
 // over the picks); 1: sqrt(softplus) + bias; 2: sigmoid + bias.  sel = value compared, score = value that becomes the
 // weight.  K rounds of argmax: the largest key by a DPP reduction, then the lowest lane holding it (a ballot) and that
 // lane's lowest expert with it: ties go to the lower expert id.
+// score and selection key of one expert for the bias modes (1: sqrt(softplus), 2: sigmoid)
+template <int MODE> __device__ __forceinline__ void bias_score(float v, float b, float& score, uint32_t& key)
+{
+    score = MODE == 1 ? sqrtf(v > 20.f ? v : log1pf(expf(v))) : 1.f / (1.f + expf(-v));
+    const float sel = score + b;
+    key = sel != sel ? 1u : max(fkey(sel), 1u);          // a NaN never wins over a number; -inf still ranks above "absent"
+}
+
+// pre = scores and keys of all lane * PER + i already worked out (LDS arrays of 64 * PER entries), or null
 template <int MODE, int PER, typename IT>
 __device__ __forceinline__ void route_row(const float* __restrict__ x, const float* __restrict__ bias, IT* __restrict__ idx,
-                                          float* __restrict__ w, int E, int K, float scale, int lane)
+                                          float* __restrict__ w, int E, int K, float scale, int lane, const float* pre_score = nullptr,
+                                          const uint32_t* pre_key = nullptr)
 {
     float score[PER];
     uint32_t key[PER];                                   // 0 = not a candidate (absent, taken, or NaN)
     const int e0 = lane * PER;
-    if (MODE == 0) {
+    if (MODE != 0 && pre_score) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) { score[i] = pre_score[e0 + i]; key[i] = pre_key[e0 + i]; }
+    } else if (MODE == 0) {
         float xv[PER], m = -INFINITY;
 #pragma unroll
         for (int i = 0; i < PER; ++i) { xv[i] = e0 + i < E ? x[e0 + i] : -INFINITY; m = fmaxf(m, xv[i]); }
@@ -69,12 +82,7 @@ __device__ __forceinline__ void route_row(const float* __restrict__ x, const flo
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             score[i] = 0.f; key[i] = 0u;
-            if (e0 + i < E) {
-                const float v = x[e0 + i];
-                score[i] = MODE == 1 ? sqrtf(v > 20.f ? v : log1pf(expf(v))) : 1.f / (1.f + expf(-v));
-                const float sel = score[i] + bias[e0 + i];
-                key[i] = sel != sel ? 1u : max(fkey(sel), 1u);      // a NaN never wins over a number; -inf still ranks above "absent"
-            }
+            if (e0 + i < E) bias_score<MODE>(x[e0 + i], bias[e0 + i], score[i], key[i]);
         }
     }
     float mine = 0.f, sum = 0.f;                          // lane k keeps pick k
@@ -109,9 +117,35 @@ __global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ log
     const int row = blockIdx.x;
     route_row<MODE, PER, IT>(logits + (int64_t)row * ld, bias, idx + (int64_t)row * K, w + (int64_t)row * K, E, K, scale, threadIdx.x);
 }
+// The bias modes spend most of their time in the transcendental functions (softplus, sqrt: ~70 instructions an expert, eight or
+// sixteen experts a lane).  Four waves share that part, one expert per thread and round, and hand the scores to the first wave
+// through LDS; the selection is the one-wave routine above.  Same functions on the same inputs: the same bits.
+template <int MODE, int PER, typename IT>
+__global__ __launch_bounds__(256) void route_kernel_mw(const float* __restrict__ logits, int64_t ld, const float* __restrict__ bias, IT* __restrict__ idx,
+                                                       float* __restrict__ w, int T, int E, int K, float scale)
+{
+    __shared__ float s_score[64 * PER];
+    __shared__ uint32_t s_key[64 * PER];
+    const int row = blockIdx.x;
+    const float* x = logits + (int64_t)row * ld;
+    for (int e = threadIdx.x; e < 64 * PER; e += 256) {
+        float sc = 0.f; uint32_t ky = 0u;
+        if (e < E) bias_score<MODE>(x[e], bias[e], sc, ky);
+        s_score[e] = sc; s_key[e] = ky;
+    }
+    __syncthreads();
+    if (threadIdx.x < 64)
+        route_row<MODE, PER, IT>(x, bias, idx + (int64_t)row * K, w + (int64_t)row * K, E, K, scale, threadIdx.x, s_score, s_key);
+}
 template <int MODE, typename IT>
 void launch_route(const float* logits, int64_t ld, const float* bias, IT* idx, float* w, int T, int E, int K, float scale, hipStream_t st)
 {
+    if constexpr (MODE != 0) {
+        if (E <= 256) route_kernel_mw<MODE, 4, IT><<<T, 256, 0, st>>>(logits, ld, bias, idx, w, T, E, K, scale);
+        else if (E <= 512) route_kernel_mw<MODE, 8, IT><<<T, 256, 0, st>>>(logits, ld, bias, idx, w, T, E, K, scale);
+        else route_kernel_mw<MODE, 16, IT><<<T, 256, 0, st>>>(logits, ld, bias, idx, w, T, E, K, scale);
+        return;
+    }
     if (E <= 256) route_kernel<MODE, 4, IT><<<T, 64, 0, st>>>(logits, ld, bias, idx, w, T, E, K, scale);
     else if (E <= 512) route_kernel<MODE, 8, IT><<<T, 64, 0, st>>>(logits, ld, bias, idx, w, T, E, K, scale);
     else route_kernel<MODE, 16, IT><<<T, 64, 0, st>>>(logits, ld, bias, idx, w, T, E, K, scale);
