@@ -87,20 +87,61 @@ __device__ __forceinline__ void route_row(const float* __restrict__ x, const flo
     }
     float mine = 0.f, sum = 0.f;                          // lane k keeps pick k
     int mine_id = 0;
-    for (int k = 0; k < K; ++k) {
-        uint32_t bk = 0u; int bi = 0;
+    if constexpr (PER == 4 || PER == 8) {
+        // Every lane sorts its own candidates once (a fixed compare-exchange network on 64-bit words: key above, PER - 1 - i below,
+        // so equal keys keep the lower expert first); a round is then the wave's largest head, the lowest lane that holds it, and
+        // that lane dropping its head.  A third of the instructions per round of scanning the lane's candidates every round,
+        // and the same picks: same keys, ties to the lowest lane and there to the lowest i.
+        uint64_t q[PER];
 #pragma unroll
-        for (int i = PER - 1; i >= 0; --i) if (key[i] >= bk) { bk = key[i]; bi = i; }   // lowest i among equals
-        const uint32_t wk = wave_umax(bk);
-        const uint64_t bal = __builtin_amdgcn_ballot_w64(bk == wk);
-        const int wl = __builtin_ctzll(bal);               // lowest lane = lowest expert ids
-        const int wi = __builtin_amdgcn_readlane(bi, wl);
-        float sc = 0.f;
+        for (int i = 0; i < PER; ++i) q[i] = ((uint64_t)key[i] << 32) | (uint32_t)(PER - 1 - i);
+        auto cx = [&](int i, int j) {                      // larger first
+            const bool sw = q[j] > q[i];
+            const uint64_t hi = sw ? q[j] : q[i], lo = sw ? q[i] : q[j];
+            q[i] = hi; q[j] = lo;
+        };
+        if constexpr (PER == 8) {
+            cx(0, 1); cx(2, 3); cx(4, 5); cx(6, 7); cx(0, 2); cx(1, 3); cx(4, 6); cx(5, 7); cx(1, 2); cx(5, 6); cx(0, 4); cx(3, 7);
+            cx(1, 5); cx(2, 6); cx(1, 4); cx(3, 6); cx(2, 4); cx(3, 5); cx(3, 4);
+        } else {
+            cx(0, 1); cx(2, 3); cx(0, 2); cx(1, 3); cx(1, 2);
+        }
+        uint32_t mine_key = 0u;
+        for (int k = 0; k < K; ++k) {
+            const uint32_t bk = (uint32_t)(q[0] >> 32);
+            const uint32_t wk = wave_umax(bk);
+            const uint64_t bal = __builtin_amdgcn_ballot_w64(bk == wk);
+            const int wl = __builtin_ctzll(bal);           // lowest lane = lowest expert ids
+            const int wi = PER - 1 - __builtin_amdgcn_readlane((int)(uint32_t)q[0], wl);
+            if (lane == k) { mine_key = wk; mine_id = wl * PER + wi; }
+            const bool win = lane == wl;
 #pragma unroll
-        for (int i = 0; i < PER; ++i) if (lane == wl && i == wi) { sc = score[i]; key[i] = 0u; }
-        sc = readlane_f(sc, wl);
-        sum += sc;
-        if (lane == k) { mine = sc; mine_id = wl * PER + wi; }
+            for (int i = 0; i + 1 < PER; ++i) q[i] = win ? q[i + 1] : q[i];
+            q[PER - 1] = win ? 0ull : q[PER - 1];
+        }
+        // the pick's score: the key read backwards (softmax: the key orders the score itself), else the expert's score again
+        if (MODE == 0) mine = __uint_as_float((mine_key & 0x80000000u) ? (mine_key & 0x7fffffffu) : ~mine_key);
+        else if (lane < K) {
+            if (pre_score) mine = pre_score[mine_id];
+            else { uint32_t ky; bias_score<MODE>(x[mine_id], bias[mine_id], mine, ky); }
+        }
+        for (int k = 0; k < K; ++k) sum += readlane_f(mine, k);          // in pick order
+    } else {
+        for (int k = 0; k < K; ++k) {
+            uint32_t bk = 0u; int bi = 0;
+#pragma unroll
+            for (int i = PER - 1; i >= 0; --i) if (key[i] >= bk) { bk = key[i]; bi = i; }   // lowest i among equals
+            const uint32_t wk = wave_umax(bk);
+            const uint64_t bal = __builtin_amdgcn_ballot_w64(bk == wk);
+            const int wl = __builtin_ctzll(bal);               // lowest lane = lowest expert ids
+            const int wi = __builtin_amdgcn_readlane(bi, wl);
+            float sc = 0.f;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) if (lane == wl && i == wi) { sc = score[i]; key[i] = 0u; }
+            sc = readlane_f(sc, wl);
+            sum += sc;
+            if (lane == k) { mine = sc; mine_id = wl * PER + wi; }
+        }
     }
     if (lane < K) {
         idx[lane] = (IT)mine_id;
