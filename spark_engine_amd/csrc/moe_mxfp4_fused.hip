@@ -281,15 +281,14 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
         if (wave == 0 && rg == 0) he[c] = e;
         __syncthreads();
         // ---- hand the rows' 32 codes + scale to every column block's copy of h (device-coherent: the readers sit on all XCDs)
-        const int per = grp.n * 9;
-        for (int u = tid; u < a.NBD * per; u += NT) {
-            const int q = u / per, rem = u % per, cc = rem / 9, w = rem % 9;
-            const int64_t row = (int64_t)q * a.P + rows[cc];
-            if (w < 8) {
-                uint32_t word = hbw[cc][w];
-                if (word == EMPTY) word = 0xffffff7fu;
-                st_dev32(a.hc + row * (I >> 2) + jb * 8 + w, word);
-            } else st_dev32(a.hsw + row * (I >> 5) + jb, he[cc]);
+        // eight threads per column block (one code word each) and one thread per column block for the scale word, row after row:
+        // no index arithmetic beyond shifts on the way out
+        for (int cc = 0; cc < grp.n; ++cc) {
+            const int pr = rows[cc];
+            uint32_t word = hbw[cc][tid & 7];
+            if (word == EMPTY) word = 0xffffff7fu;
+            for (int q = tid >> 3; q < a.NBD; q += NT / 8) st_dev32(a.hc + ((int64_t)q * a.P + pr) * (I >> 2) + jb * 8 + (tid & 7), word);
+            for (int q = tid; q < a.NBD; q += NT) st_dev32(a.hsw + ((int64_t)q * a.P + pr) * (I >> 5) + jb, he[cc]);
         }
         TRACE(5);
     }
