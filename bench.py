@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 FP8_PEAK_TFLOPS = 5000.0       # MI355X published dense FP8 matrix rate (the block-scaled FP8 x FP4 products run at it)
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known
 # size); filled in from the committed counter summaries, None where no counter run exists
-TRAFFIC = {("c2", 1): 19782587, ("c3", 1): 99324319, ("c5", 1): 6406405504}
+TRAFFIC = {("c2", 1): 19782641, ("c3", 1): 99177977, ("c5", 1): 6406407843}
 
 
 def parse():
