@@ -135,21 +135,20 @@ __device__ __forceinline__ int ld_idx_k(const void* idx, int itype, int i) { ret
 
 struct Group { int e, n; };
 // item g of the call: expert and its pair rows (ascending) in rows[], or n = 0 when the call has fewer items.  All threads
-// call; wave 0 works the item out (one barrier).  Leaves every pair's expert in sidx[] when R > 1.
-__device__ __forceinline__ Group find_item(const FArgs& a, int g, int* sidx, int* owner, int* rows, int* misc)
+// call; wave 0 works the item out (one barrier).
+__device__ __forceinline__ Group find_item(const FArgs& a, int g, int* owner, int* rows, int* misc)
 {
     const int P = a.P, tid = threadIdx.x;
     if (a.R == 1) {                                       // every pair is its own item
         if (g >= P) return Group{0, 0};
+        const int e = ld_idx_k(a.idx, a.c.itype, g);      // on its way while the block meets at the barrier
         if (tid == 0) rows[0] = g;
         __syncthreads();
-        return Group{ld_idx_k(a.idx, a.c.itype, g), 1};
+        return Group{e, 1};
     }
     if (tid < 64) {
         WaveItems<PF_MAX / 64> wi;
         wave_items_init(wi, P, tid, owner, [&](int p) { return exl3_ld_idx(a.idx, a.c.itype, p); });
-#pragma unroll
-        for (int j = 0; j < PF_MAX / 64; ++j) if (tid + 64 * j < P) sidx[tid + 64 * j] = wi.e[j];
         int n = 0;
         const int e = wave_items_pick(wi, g, tid, rows, n);
         if (tid == 0) { misc[0] = e; misc[1] = n; }
@@ -163,7 +162,7 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
 {
     __shared__ __align__(16) uint16_t xs[MR][FW * TWMAX * 16];   // this block's K slice of the transformed activations (fp16)
     __shared__ float red[FW][MR][128];
-    __shared__ int sidx[PF_MAX], rows[RF_MAX], misc[4];
+    __shared__ int rows[RF_MAX], misc[4];
     __shared__ int owner[EMAX_F];                         // one int per expert id: scratch of the item lookup
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bid = blockIdx.x;
@@ -198,7 +197,7 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
     }
     if (tid == 0) misc[2] = 1;
     Group grp{0, 0};
-    if (g >= 0) grp = find_item(a, g, sidx, owner, rows, misc);
+    if (g >= 0) grp = find_item(a, g, owner, rows, misc);
     TRACE(1);
     if (isC) {
         if (s) {
