@@ -214,6 +214,8 @@ SPARK_API void spark_debug_exl3_trace(long long* buf);
 SPARK_API void spark_debug_mx_trace(long long* buf);
 /* exchange mode of the single-launch EXL3 kernel: 1 = same-XCD through L2, 0 = device-coherent, -1 = measure placement again */
 SPARK_API void spark_debug_exl3_local(int v);
+/* the same switch for the single-launch MXFP4 kernel */
+SPARK_API void spark_debug_mx_local(int v);
 /* k-tiles per wave of a stage-1 block of the single-launch EXL3 kernel: 4 or 8 forces it, 0 = chosen by the shape (the default) */
 SPARK_API void spark_debug_exl3_twa(int v);
 

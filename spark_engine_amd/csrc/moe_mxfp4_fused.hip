@@ -587,6 +587,8 @@ int mx_fused_launch(const void* x, const void* xs, int R, const int64_t* idx, co
 // diagnostics: device buffer of 16 time stamps (100 MHz) per block of the next launches, or null (recorded by builds with
 // -DSPK_MX_TRACE only)
 extern "C" __attribute__((visibility("default"))) void spark_debug_mx_trace(long long* buf) { g_trace = buf; }
+// diagnostics: force the exchange mode of the single-launch path (1 same-XCD through L2, 0 device-coherent, -1 measure placement again)
+extern "C" __attribute__((visibility("default"))) void spark_debug_mx_local(int v) { g_local = v; }
 
 }  // namespace mx
 }  // namespace spk

@@ -239,3 +239,23 @@ def test_ds41_two_bit_coded_scales(ops, oracle):
         ops.moe_s2_set(False)
     assert np.array_equal(host(y2_s2), host(y2_raw))
     assert rel_l2(host(y2_s2), oracle.mxfp4_moe(x2, idx2, rw2, *ws)) <= TOL
+
+
+@pytest.mark.parametrize("R", [1, 4])
+def test_device_coherent_exchange_gives_the_same_bits(ops, oracle, R):
+    # the single-launch kernel hands the per-pair outputs over inside one XCD's L2 where the placement check allows and through
+    # device-coherent accesses otherwise: the fallback is forced here and must not change a bit
+    H, I, E, topk, ns = 1024, 512, 12, 6, 1
+    g = synth.rng(260 + R)
+    ws, x, idx, rw = _case(g, R, H, I, E, topk, ns)
+    ex = ops.Mxfp4Experts(*[dev(a) for a in ws], n_shared=ns)
+    L = ops._lib()
+    try:
+        L.spark_debug_mx_local(0)
+        a = host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex))
+        L.spark_debug_mx_local(-1)                                       # measure the placement again on the next workspace set-up
+        b = host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ex))
+    finally:
+        L.spark_debug_mx_local(-1)
+    assert rel_l2(a, oracle.mxfp4_moe(x, idx, rw, *ws, n_shared=ns)) <= TOL
+    assert np.array_equal(a, b)
