@@ -305,6 +305,11 @@ SPARK_API int spark_exl3_moe_path(int R, int H, int I, int E, int topk, int flag
 /* diagnostics: the most rows (0..8) a call may have to run as the single launch where the MXFP4 grouped GEMM could take it too;
  * negative = the built-in rule (8 on T16 records; 2 on the reference's tile layouts, 4 from an intermediate width of 1536 on) */
 SPARK_API void spark_debug_mx_fused_rows(int rows);
+/* Where the several-kernel MXFP4 path (flags bit 1 of spark_mxfp4_moe_x; every call of more than 8 rows) left the act-quantised
+ * intermediate of its last call inside a spark_mxfp4_moe* workspace: E4M3 codes hq [P, I] and UE8M0 scale bytes hs [P, I / 32] in
+ * grouped order, prow [P] = the pair (row * (topk + n_shared) + slot) of each grouped row.  For tests that compare the
+ * intermediate with the CPU oracle's; returns 1 on a shape the entry points refuse. */
+SPARK_API int spark_debug_mx_ws_h(void* ws, int R, int H, int I, int topk, int E, int n_shared, void** hq, void** hs, int** prow);
 /* k-tiles per wave of a stage-1 block of the single-launch EXL3 kernel: 4 or 8 forces it, 0 = chosen by the shape (the default) */
 SPARK_API void spark_debug_exl3_twa(int v);
 

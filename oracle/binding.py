@@ -44,7 +44,8 @@ def _load():
         "orc_act_quant_fp8": (None, [vp, vp, vp, i64]), "orc_act_quant32": (None, [vp, vp, i64]),
         "orc_swiglu_quant": (None, [vp, vp, i32, i32, f32]), "orc_silu_mul": (None, [vp, vp, vp, i32]),
         "orc_gate_scale": (None, [vp, i64, i32, vp, vp, i32, i32]),
-        "orc_mxfp4_moe": (None, [vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp]),
+        "orc_mxfp4_moe": (None, [vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp]),
+        "orc_mxfp4_moe_from_h": (None, [vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, vp, vp]),
         "orc_mxfp4_gemv": (None, [vp, vp, vp, vp, i32, i32, i32]),
         "orc_fp8_block_gemv": (None, [vp, vp, vp, vp, i32, i32, i32, i32]),
         "orc_fp8_e8m0_gemv": (None, [vp, vp, vp, vp, i32, i32, i32]),
@@ -251,8 +252,10 @@ def gate_scale(gl, col, d):
     return out
 
 
-def mxfp4_moe(x_bits, idx, rw, w1, s1, w3, s3, w2, s2, n_shared=0, add=None, want_pairs=False):
-    """Stacked natural-layout weights [E(+n_shared), ...]; x bf16 bits [R, H]."""
+def mxfp4_moe(x_bits, idx, rw, w1, s1, w3, s3, w2, s2, n_shared=0, add=None, want_pairs=False, want_h=False):
+    """Stacked natural-layout weights [E(+n_shared), ...]; x bf16 bits [R, H].  want_h: also the act-quantised intermediate of
+    every pair (routed pairs first, then the shared ones): E4M3 codes [P + R * n_shared, I], scale bytes [.., I / 32] and each
+    element's rounding margin [.., I] (the relative error of its sums or product it takes to change one of its bf16 roundings)."""
     x_bits, idx, rw = _c(x_bits, np.uint16), _c(idx, np.int64), _c(rw, np.float32)
     arrs = [_c(a, np.uint8) for a in (w1, s1, w3, s3, w2, s2)]
     R, H = x_bits.shape
@@ -261,10 +264,29 @@ def mxfp4_moe(x_bits, idx, rw, w1, s1, w3, s3, w2, s2, n_shared=0, add=None, wan
     E = arrs[0].shape[0] - n_shared
     y = np.empty((R, H), np.float32)
     pairs = np.empty((R * topk, H), np.float32) if want_pairs else None
+    hq = np.empty((R * (topk + n_shared), I), np.uint8) if want_h else None
+    hs = np.empty((R * (topk + n_shared), I // 32), np.uint8) if want_h else None
+    hm = np.empty((R * (topk + n_shared), I), np.float32) if want_h else None
     if add is not None:
         add = _c(add, np.float32)
-    lib.orc_mxfp4_moe(_p(x_bits), R, _p(idx), _p(rw), *[_p(a) for a in arrs], H, I, topk, E, n_shared, _p(add), _p(y), _p(pairs))
-    return (y, pairs) if want_pairs else y
+    lib.orc_mxfp4_moe(_p(x_bits), R, _p(idx), _p(rw), *[_p(a) for a in arrs], H, I, topk, E, n_shared, _p(add), _p(y), _p(pairs), _p(hq), _p(hs), _p(hm))
+    out = (y,) + ((pairs,) if want_pairs else ()) + ((hq, hs, hm) if want_h else ())
+    return out if len(out) > 1 else y
+
+
+def mxfp4_moe_from_h(hq, hs, idx, w2, s2, n_shared=0, add=None):
+    """The down products and the sum of a given intermediate (codes hq [R * topk + R * n_shared, I], scale bytes hs, pairs ordered as
+    mxfp4_moe(want_h=True) returns them); w2, s2 stacked [E + n_shared, H, ...]."""
+    hq, hs, idx = _c(hq, np.uint8), _c(hs, np.uint8), _c(idx, np.int64)
+    w2, s2 = _c(w2, np.uint8), _c(s2, np.uint8)
+    R, topk = idx.shape
+    H, I = w2.shape[1], w2.shape[2] * 2
+    E = w2.shape[0] - n_shared
+    y = np.empty((R, H), np.float32)
+    if add is not None:
+        add = _c(add, np.float32)
+    lib.orc_mxfp4_moe_from_h(_p(hq), _p(hs), R, _p(idx), _p(w2), _p(s2), H, I, topk, E, n_shared, _p(add), _p(y))
+    return y
 
 
 def mxfp4_gemv(x_bits, w, s):

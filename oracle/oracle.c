@@ -515,18 +515,55 @@ EXPORT void orc_gate_scale(const float* gl, int64_t ldg, int col, const float* d
 
 /* ------------------------------------------------------------------ DeepSeek MXFP4 MoE ------------ */
 
-/* One pair: out[H] = w2 . q(bf16(silu(min(bf16(w1.x),10)) * clamp(bf16(w3.x),+-10) * rw)), dequantise + fp32 matmul.
+/* Dot products whose result a quantiser reads (gate / up: rounded to bf16, then act_quant): summed in binary64 and rounded
+ * once to binary32.  The reference's moe_ref leaves the order of this sum to its BLAS (x.matmul, ds41/kern.rs:1124-1125); the
+ * exact sum is the value every binary32 order approximates, and a binary64 sum of these terms (products of a 4-bit and a 6-bit
+ * significand, a few thousand of them) is that value to 1e-16.  With binary32 sums here the oracle's own summation error (5e-7 of
+ * the sum, eight chains of K / 8 terms) decided more bf16 / E4M3 roundings of the intermediate than the kernels' did. */
+static void gemv_nk_f64acc(const float* x, const float* W, int N, int K, float* y, double* yd, double* ynorm)
+{
+    /* yd, ynorm (optional): the binary64 sums and the Euclidean norm of each sum's terms (the size of its partial sums: what a
+     * binary32 summation's error is relative to) */
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < N; ++n) {
+        const float* wr = W + (size_t)n * K;
+        double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, sq = 0.0;
+        for (int k = 0; k < K; k += 8)
+            for (int j = 0; j < 8; ++j) { const double p = (double)x[k + j] * (double)wr[k + j]; acc[j] += p; sq += p * p; }
+        const double t = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+        y[n] = (float)t;
+        if (yd) { yd[n] = t; ynorm[n] = sqrt(sq); }
+    }
+}
+/* Distance of v from the nearest point where its rounding to bf16 changes (the midpoint between neighbouring bf16 values on the
+ * side of bf16(v) that v lies on): how large an error of v it takes to move bf16(v). */
+static double bf16_margin(double v)
+{
+    const double r = (double)bf16r((float)v);
+    int ex;
+    (void)frexp(r != 0.0 ? r : (v != 0.0 ? v : 1.0), &ex);    /* |r| in [2^(ex-1), 2^ex): one step of bf16 there is 2^(ex-8) */
+    double half = ldexp(1.0, ex - 9);
+    if (fabs(v) < fabs(r) && fabs(r) == ldexp(1.0, ex - 1)) half *= 0.5;   /* below a power of two the steps are half as wide */
+    return fabs(fabs(v - r) - half);
+}
+/* One pair: out[H] = w2 . q(bf16(silu(min(bf16(w1.x),10)) * clamp(bf16(w3.x),+-10) * rw)), dequantise + matmul.
  * xd: the act-quantized input as binary32 [H].  w1/w3 [I, H/2]+[I, H/32], w2 [H, I/2]+[H, I/32] of ONE expert.
+ * hq / hs (optional): the intermediate's E4M3 codes [I] and UE8M0 scale bytes [I / 32]; margin (optional) [I]: the smallest
+ * bf16_margin of the element's three roundings, each relative to the size of what is rounded (gate sum and up sum: the norm of the
+ * sum's terms; the product: itself), i.e. how close the element is to coming out differently under another order of the binary32
+ * sums or another library's expf.
  * reference ds41/kern.rs:1116-1133 (moe_ref), ds41_moe.cu:1-6,161-181. */
 static void ds41_pair(const float* xd, const uint8_t* w1, const uint8_t* s1, const uint8_t* w3, const uint8_t* s3, const uint8_t* w2,
-                      const uint8_t* s2, int H, int I, float rw, float* W, float* out)
+                      const uint8_t* s2, int H, int I, float rw, float* W, float* out, uint8_t* hq, uint8_t* hs, float* margin)
 {
     float* g = (float*)malloc((size_t)I * 4 * 3);
     float *u = g + I, *hm = u + I;
+    double* gd = margin ? (double*)malloc((size_t)I * 8 * 4) : NULL;
+    double *ud = gd ? gd + I : NULL, *gn = gd ? gd + 2 * I : NULL, *un = gd ? gd + 3 * I : NULL;
     orc_mxfp4_dequant(w1, s1, I, H, W);
-    orc_gemv_nk(xd, W, 1, I, H, g);
+    gemv_nk_f64acc(xd, W, I, H, g, gd, gn);
     orc_mxfp4_dequant(w3, s3, I, H, W);
-    orc_gemv_nk(xd, W, 1, I, H, u);
+    gemv_nk_f64acc(xd, W, I, H, u, ud, un);
     uint16_t hb[32];
     for (int j0 = 0; j0 < I; j0 += 32) {
         float a = 0.f;
@@ -536,14 +573,24 @@ static void ds41_pair(const float* xd, const uint8_t* w1, const uint8_t* s1, con
             const float y = bf16r(silu(gt) * up * rw);
             hb[j] = orc_f32_to_bf16(y);
             a = fmaxf(a, fabsf(y));
+            if (margin) {
+                const double yd = (double)gt / (1.0 + exp(-(double)gt)) * (double)up * (double)rw;
+                const double mg = gn[j0 + j] > 0.0 ? bf16_margin(gd[j0 + j]) / gn[j0 + j] : 1.0, mu = un[j0 + j] > 0.0 ? bf16_margin(ud[j0 + j]) / un[j0 + j] : 1.0;
+                margin[j0 + j] = (float)fmin(fmin(mg, mu), yd != 0.0 ? bf16_margin(yd) / fabs(yd) : 1.0);
+            }
         }
         const uint8_t e = orc_aq_scale(a);
         const float sc = u2f((uint32_t)e << 23);
-        for (int j = 0; j < 32; ++j) hm[j0 + j] = orc_e4m3_to_f32(orc_aq_byte(orc_bf16_to_f32(hb[j]), e)) * sc;
+        if (hs) hs[j0 / 32] = e;
+        for (int j = 0; j < 32; ++j) {
+            const uint8_t q = orc_aq_byte(orc_bf16_to_f32(hb[j]), e);
+            if (hq) hq[j0 + j] = q;
+            hm[j0 + j] = orc_e4m3_to_f32(q) * sc;
+        }
     }
     orc_mxfp4_dequant(w2, s2, H, I, W);
     orc_gemv_nk(hm, W, 1, H, I, out);
-    free(g);
+    free(g); free(gd);
 }
 /* Routed MXFP4 experts.  x bf16 [R, H] (NOT yet quantized: act_quant per 32 is applied here, as the layer does before
  * the experts, reference ds41/kern.rs act_quant_fp8 + moe_mx).  Stacked natural-layout weights w1,w3 [E, I, H/2],
@@ -553,9 +600,10 @@ static void ds41_pair(const float* xd, const uint8_t* w1, const uint8_t* s1, con
  * first, then added to add).  pair_out (optional) receives the per-pair outputs [R*topk, H]. */
 EXPORT void orc_mxfp4_moe(const uint16_t* x, int R, const int64_t* idx, const float* rw, const uint8_t* w1, const uint8_t* s1,
                           const uint8_t* w3, const uint8_t* s3, const uint8_t* w2, const uint8_t* s2, int H, int I, int topk, int E,
-                          int n_shared, const float* add, float* y, float* pair_out)
+                          int n_shared, const float* add, float* y, float* pair_out, uint8_t* h_codes, uint8_t* h_scales, float* h_margin)
 {
-    (void)E;
+    /* h_codes [R * topk + R * n_shared, I], h_scales [.., I / 32], h_margin [.., I] (optional): the act-quantised intermediate of
+     * every pair and each element's rounding margin (ds41_pair), the routed pairs (r, k) first, then the shared ones (r, j) */
     const int P = R * topk;
     float* xd = (float*)malloc((size_t)R * H * 4);
     {
@@ -571,13 +619,15 @@ EXPORT void orc_mxfp4_moe(const uint16_t* x, int R, const int64_t* idx, const fl
     for (int p = 0; p < P; ++p) {
         const int64_t e = idx[p];
         ds41_pair(xd + (size_t)(p / topk) * H, w1 + e * wsz, s1 + e * ssz, w3 + e * wsz, s3 + e * ssz, w2 + e * wsz, s2 + e * ssz, H, I, rw[p], W,
-                  out + (size_t)p * H);
+                  out + (size_t)p * H, h_codes ? h_codes + (size_t)p * I : NULL, h_scales ? h_scales + (size_t)p * (I / 32) : NULL,
+                  h_margin ? h_margin + (size_t)p * I : NULL);
     }
     for (int r = 0; r < R; ++r)
         for (int j = 0; j < n_shared; ++j) {
             const int64_t e = E + j;
+            const size_t q = (size_t)P + (size_t)r * n_shared + j;
             ds41_pair(xd + (size_t)r * H, w1 + e * wsz, s1 + e * ssz, w3 + e * wsz, s3 + e * ssz, w2 + e * wsz, s2 + e * ssz, H, I, 1.0f, W,
-                      out + (size_t)(P + r * n_shared + j) * H);
+                      out + q * H, h_codes ? h_codes + q * I : NULL, h_scales ? h_scales + q * (I / 32) : NULL, h_margin ? h_margin + q * I : NULL);
         }
     for (int r = 0; r < R; ++r)
         for (int n = 0; n < H; ++n) {
@@ -589,6 +639,33 @@ EXPORT void orc_mxfp4_moe(const uint16_t* x, int R, const int64_t* idx, const fl
         }
     if (pair_out) memcpy(pair_out, out, (size_t)P * H * 4);
     free(out); free(W); free(xd);
+}
+/* The second half of the layer alone: the down products of a GIVEN act-quantised intermediate (codes h_codes [R * topk + R * n_shared, I]
+ * and scale bytes h_scales [.., I / 32], pairs ordered as orc_mxfp4_moe hands them out) and the sum in the reference's order
+ * (ds41_mx.cu:302-317).  Lets a test hold a kernel's output against the oracle evaluated on the kernel's own intermediate. */
+EXPORT void orc_mxfp4_moe_from_h(const uint8_t* h_codes, const uint8_t* h_scales, int R, const int64_t* idx, const uint8_t* w2, const uint8_t* s2,
+                                 int H, int I, int topk, int E, int n_shared, const float* add, float* y)
+{
+    const int P = R * topk, Q = P + R * n_shared;
+    float* W = (float*)malloc((size_t)H * I * 4);
+    float* hm = (float*)malloc((size_t)I * 4);
+    float* out = (float*)malloc((size_t)(Q > 0 ? Q : 1) * H * 4);
+    const size_t wsz = (size_t)I * H / 2, ssz = (size_t)I * H / 32;
+    for (int q = 0; q < Q; ++q) {
+        const int64_t e = q < P ? idx[q] : E + (q - P) % n_shared;
+        for (int j = 0; j < I; ++j) hm[j] = orc_e4m3_to_f32(h_codes[(size_t)q * I + j]) * u2f((uint32_t)h_scales[(size_t)q * (I / 32) + j / 32] << 23);
+        orc_mxfp4_dequant(w2 + e * wsz, s2 + e * ssz, H, I, W);
+        orc_gemv_nk(hm, W, 1, H, I, out + (size_t)q * H);
+    }
+    for (int r = 0; r < R; ++r)
+        for (int n = 0; n < H; ++n) {
+            float acc = add ? add[(size_t)r * H + n] : 0.f;
+            for (int j = 0; j < n_shared; ++j) acc += out[(size_t)(P + r * n_shared + j) * H + n];
+            float s = 0.f;
+            for (int k = 0; k < topk; ++k) s += out[(size_t)(r * topk + k) * H + n];
+            y[(size_t)r * H + n] = acc + s;
+        }
+    free(out); free(hm); free(W);
 }
 
 /* ------------------------------------------------------------------ dense GEMVs ------------------- */

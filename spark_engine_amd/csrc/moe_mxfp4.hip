@@ -6,15 +6,18 @@
 // Semantics: reference engine-rs/shim/ds41_moe.cu:1-24 and ds41_mx.cu:1-16,95-317,1436-1523 (ds41_moe_mx_ex),
 // reference engine-rs/src/ds41/kern.rs:1116-1133 (moe_ref).
 //
-// MI355X design.  The products run on the block-scaled matrix unit, v_mfma_scale_f32_16x16x128_f8f6f4 with A = 16 weight
-// rows in E2M1 (one E8M0 scale per lane = per row and 32-block, exactly the stored format) and B = up to 16 token rows in
-// E4M3 with their UE8M0 scales.  A lane's A operand is 16 contiguous bytes of the weight stream, so the packed weights go
-// from the 128-bit load straight into the instruction with no unpacking; products and scales are exact, only the
-// summation order differs from a dequantize + FP32 matmul.
+// MI355X design.  A lane's piece of the weight stream is 16 contiguous bytes = the 32 E2M1 codes of one scale block of one row.
+// The down product runs on the block-scaled matrix unit, v_mfma_scale_f32_16x16x128_f8f6f4, with A = 16 weight rows in E2M1 (one
+// E8M0 scale per lane = per row and 32-block, exactly the stored format) and B = up to 16 token rows in E4M3 with their UE8M0
+// scales: the packed weights go from the 128-bit load straight into the instruction.  That instruction aligns the products of a
+// 32-block to the block's largest and drops what lies about 14 bits under it (1e-5 of a sum), which is harmless for the down
+// product but not for gate / up, whose sums are rounded to bf16 and quantised: those run on v_mfma_f32_16x16x32_bf16 with both
+// operands converted exactly (moe_mxfp4.hpp: mfma_exact_step), four instructions per 128-wide step, dword j of the same 16 bytes
+// feeding instruction j.
 // Operand layout measured on gfx950: A/B lane l = row/column l % 16, K group g = l / 16.  An E2M1 operand holds
 // k = 32 g + e (nibble e of its 16 bytes); an E4M3 operand holds k = 16 g + e in registers 0-3 and k = 64 + 16 g + e in
 // registers 4-7; the scale byte of lane l applies to logical block g (k in [32 g, 32 g + 32)); D lane l = column l % 16,
-// rows 4 (l / 16) + {0..3}.
+// rows 4 (l / 16) + {0..3}.  v_mfma_f32_16x16x32_bf16: lane l = row/column l % 16, k = 8 (l / 16) + {0..7}, D as above.
 //
 // Weight storage ("T16" records, written once by spark_mxfp4_prepack): per 16 rows and 512-wide K group one record of
 // 4352 bytes = 4 steps x (64 lanes x 16 bytes of codes) + 64 lanes x 4 scale bytes (byte s = step s).  A wave streams a
@@ -195,10 +198,9 @@ __global__ __launch_bounds__(64 * UP_WAVES) void up_kernel(const uint8_t* __rest
             for (int s = 0; s < 4; ++s) {
                 const int step = kg * 4 + s;
                 if (step >= steps) break;
-                v8i b; uint32_t sb;
-                load_b(xr, xsr, step, lane, b, sb);
+                const XOp xo = load_x(xr, xsr, step, lane);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) acc[t] = mfma_group_step(s, a[t][s], b, acc[t], sa[t], sb);
+                for (int t = 0; t < 4; ++t) acc[t] = mfma_exact_step(s, a[t][s], xo, acc[t], sa[t]);
             }
         }
 #pragma unroll
@@ -337,14 +339,9 @@ __global__ __launch_bounds__(64 * UP_WAVES, 4) void up_res_kernel(const uint8_t*
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 if (kg * 4 + s >= steps) break;
-                v8i b; uint32_t sb;
-#ifndef SPK_EXP_NOX
-                load_b(xq + (int64_t)tok * H, xs + (int64_t)tok * (H >> 5), kg * 4 + s, lane, b, sb);
-#else
-                b = v8i{tok, s, lane, cg, 1, 2, 3, 4}; sb = 127;
-#endif
+                const XOp xo = load_x(xq + (int64_t)tok * H, xs + (int64_t)tok * (H >> 5), kg * 4 + s, lane);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) acc[t] = mfma_group_step(s, a[t][s], b, acc[t], sa[t], sb);
+                for (int t = 0; t < 4; ++t) acc[t] = mfma_exact_step(s, a[t][s], xo, acc[t], sa[t]);
             }
         }
         if (cg < 3) GTRACE(2 + cg * 4);
@@ -376,14 +373,10 @@ __global__ __launch_bounds__(64 * UP_WAVES, 4) void up_res_kernel(const uint8_t*
 #pragma unroll
         for (int w = 0; w < UP_WAVES; ++w) am = fmaxf(am, amx[w][c]);
         const uint32_t e = aq_scale(am);
-#ifndef SPK_EXP_NOST
         if (valid) {
             hq[(int64_t)pos * I + j0 + 16 * tp + 4 * rg + v] = (uint8_t)aq_byte(yv, e);
             if (wave == 0 && rg == 0) hs[(int64_t)pos * (I >> 5) + (j0 >> 5)] = (uint8_t)e;
         }
-#else
-        if (valid && e == 0x12345u) hq[0] = (uint8_t)aq_byte(yv, e);
-#endif
         __syncthreads();
         pos = posn; tok = tokn; wgt = wgtn; posn = pos2; tokn = tok2; wgtn = wgt2;
     }
@@ -460,7 +453,8 @@ __global__ __launch_bounds__(64 * DN_WAVES) void down_res_kernel(const uint8_t* 
 // MFMA A operand through a four-step register ring that is refilled as soon as a step's MFMAs are issued, and results leave in
 // whole 128-byte lines.  Each K group accumulates from zero and the groups are added in order: the values are the same bits as
 // up_kernel / down_kernel and the single-launch kernel produce (reference engine-rs/shim/ds41_mx.cu:694-932 keeps the same
-// property between its grouped GEMM and its decode kernels).
+// property between its grouped GEMM and its decode kernels).  Gate / up: the exact bf16 form, the activation rows staged as finished
+// bf16 operands (xb_put); down: the block-scaled instruction on staged codes.
 constexpr int GT_ROWS = 32;            // rows of a GEMM item
 constexpr int GT_XS = 528;             // LDS stride of a staged row: one K group (512 bytes) + 16: conflict-free 16-byte reads down a column
 constexpr int GT_FEAT = 128;           // output features / columns of a block
@@ -633,18 +627,43 @@ __device__ __forceinline__ KVisit k_visit(int i, int nkg)
     }
 }
 
+// The gate / up operand of the grouped GEMM is staged as bf16: thread (row, 32-block) converts its block's 32 E4M3 codes with the
+// block's UE8M0 scale (exact) and writes 64 bytes, so that the eight waves read finished B operands of v_mfma_f32_16x16x32_bf16
+// (16 bytes a lane and instruction) instead of each converting the same codes again.  GT_XB: the row stride, 16 bytes over a multiple
+// of 256: the 16-byte reads of 16 rows at one column cover every bank once.
+constexpr int GT_XB = 1024 + 16;
+struct XStageB { uint4 x0, x1; uint32_t sb; bool in; };
+template <bool GEN>
+__device__ __forceinline__ XStageB xb_fetch(const uint8_t* xrow, const uint8_t* xsrow, int kg, int sch, int K)
+{
+    XStageB r;
+    r.in = !GEN || kg * 512 + sch * 32 < K;
+    const int off = r.in ? sch : 0;                        // past the row's end: the group's first block again (a valid address), stored as zeros
+    const uint8_t* p = xrow + kg * 512 + off * 32;
+    r.x0 = *(const uint4*)p;
+    r.x1 = *(const uint4*)(p + 16);
+    r.sb = xsrow[kg * 16 + off];
+    return r;
+}
+__device__ __forceinline__ void xb_put(const XStageB& r, unsigned char* dst)
+{
+    const uint32_t m = r.in ? ~0u : 0u;
+    const XOp o = x_operand(make_uint4(r.x0.x & m, r.x0.y & m, r.x0.z & m, r.x0.w & m), make_uint4(r.x1.x & m, r.x1.y & m, r.x1.z & m, r.x1.w & m), r.sb);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { uint4 v; __builtin_memcpy(&v, &o.b[j], 16); *(uint4*)(dst + 16 * j) = v; }
+}
+
 template <int LAYOUT, bool GEN>
 __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, WMat w1, WMat w3, int H, int I, int TT,
                                                          const int* __restrict__ G, const Item* __restrict__ items, const int* __restrict__ prow,
                                                          const float* __restrict__ pw, uint8_t* __restrict__ hq, uint8_t* __restrict__ hs)
 {
-    __shared__ __align__(16) unsigned char xl[2][GT_ROWS * GT_XS];
-    __shared__ __align__(16) unsigned char xsl[2][GT_ROWS * 16];
+    extern __shared__ __align__(16) unsigned char gsm[];  // xl [2][GT_ROWS * GT_XB], then the epilogue's hbuf [GT_ROWS][GT_FEAT + 16] over it
     __shared__ int toks[GT_ROWS];
     __shared__ float wgts[GT_ROWS];
     __shared__ float amx[8][2][16];
-    __shared__ __align__(16) unsigned char hbuf[GT_ROWS][GT_FEAT + 16];
     __shared__ __align__(4) unsigned char hes[GT_ROWS][4];
+    unsigned char* const xl = gsm;
     const Item it = items[blockIdx.y];             // requested together with the item count (entries past it hold anything)
     if ((int)blockIdx.y >= *G) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, rg = lane >> 4;
@@ -665,14 +684,14 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
     sa[0] = t1.scales_raw(0); sa[1] = t3.scales_raw(0);
     const int kg1 = k_visit<GEN, UP_WAVES>(min(1, nkg - 1), nkg).kg;
     __syncthreads();
-    // staging: thread = (row, 32-byte chunk) of a K group; threads 0..31 also carry the row's 16 scale bytes
+    // staging: thread = (row, 32-block) of a K group
     const int srow = tid >> 4, sch = tid & 15;
     const uint8_t* xrow = xq + (int64_t)toks[srow] * H;
-    const uint8_t* xsrow = xs + (int64_t)toks[tid & (GT_ROWS - 1)] * (H >> 5);
-    unsigned char* const xdst = &xl[0][srow * GT_XS + sch * 32];
-    XStage xf = x_fetch<GEN>(xrow, xsrow, 0, sch, H);
-    x_put<GEN>(xf, xdst, &xsl[0][(tid & (GT_ROWS - 1)) * 16], tid < GT_ROWS);
-    xf = x_fetch<GEN>(xrow, xsrow, kg1, sch, H);
+    const uint8_t* xsrow = xs + (int64_t)toks[srow] * (H >> 5);
+    unsigned char* const xdst = xl + srow * GT_XB + sch * 64;
+    XStageB xf = xb_fetch<GEN>(xrow, xsrow, 0, sch, H);
+    xb_put(xf, xdst);
+    xf = xb_fetch<GEN>(xrow, xsrow, kg1, sch, H);
     __syncthreads();
     v4f tot[2][2];
 #pragma unroll
@@ -680,6 +699,7 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) tot[m][rt] = v4f{0.f, 0.f, 0.f, 0.f};
     v4f cur[2][2];
+    const unsigned char* const bbase = xl + c * GT_XB + 64 * rg;
     for (int i = 0; i < nkg; ++i) {
         const KVisit vis = k_visit<GEN, UP_WAVES>(i, nkg);
         const int buf = i & 1, kn = k_visit<GEN, UP_WAVES>(min(i + 1, nkg - 1), nkg).kg;
@@ -695,18 +715,22 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
         for (int m = 0; m < 2; ++m)
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) asm volatile("" : "+v"(cur[m][rt]));
+        const unsigned char* bp = bbase + buf * (GT_ROWS * GT_XB);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const v4i a0 = ATile<LAYOUT, GEN>::fix(a[0][s]), a1 = ATile<LAYOUT, GEN>::fix(a[1][s]);
+            const float f0s = e8m0_to_f32((sc0 >> (8 * s)) & 0xffu), f1s = e8m0_to_f32((sc1 >> (8 * s)) & 0xffu);
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) {
-                if (rt < nrt) {
-                    const unsigned char* bp = &xl[buf][(rt * 16 + c) * GT_XS + s * 128 + 16 * rg];
-                    const uint4 lo = *(const uint4*)bp, hi = *(const uint4*)(bp + 64);
-                    const v8i b = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-                    const uint32_t sb = *(const uint32_t*)&xsl[buf][(rt * 16 + c) * 16 + s * 4] >> (8 * rg);
-                    cur[0][rt] = mfma_group_step(s, a0, b, cur[0][rt], sc0, sb);
-                    cur[1][rt] = mfma_group_step(s, a1, b, cur[1][rt], sc1, sb);
+            for (int j = 0; j < 4; ++j) {
+                const bf8v w0 = a_operand((uint32_t)a0[j], f0s), w1v = a_operand((uint32_t)a1[j], f1s);
+                bf8v b0, b1;
+                { const uint4 v = *(const uint4*)(bp + s * 256 + 16 * j); __builtin_memcpy(&b0, &v, 16); }
+                cur[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, b0, cur[0][0], 0, 0, 0);
+                cur[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1v, b0, cur[1][0], 0, 0, 0);
+                if (nrt > 1) {
+                    { const uint4 v = *(const uint4*)(bp + 16 * GT_XB + s * 256 + 16 * j); __builtin_memcpy(&b1, &v, 16); }
+                    cur[0][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, b1, cur[0][1], 0, 0, 0);
+                    cur[1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1v, b1, cur[1][1], 0, 0, 0);
                 }
             }
             a[0][s] = t1.codes(kn, s);                 // the ring slot is free again: the same step of the next K group
@@ -720,11 +744,12 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
         }
         sa[0] = san0; sa[1] = san1;
         // the next K group of the rows into the other buffer (nobody reads it before the barrier), the one after into registers
-        x_put<GEN>(xf, xdst + (buf ^ 1) * (GT_ROWS * GT_XS), &xsl[buf ^ 1][(tid & (GT_ROWS - 1)) * 16], tid < GT_ROWS);
-        xf = x_fetch<GEN>(xrow, xsrow, k_visit<GEN, UP_WAVES>(min(i + 2, nkg - 1), nkg).kg, sch, H);
+        xb_put(xf, xdst + (buf ^ 1) * (GT_ROWS * GT_XB));
+        xf = xb_fetch<GEN>(xrow, xsrow, k_visit<GEN, UP_WAVES>(min(i + 2, nkg - 1), nkg).kg, sch, H);
         __syncthreads();
     }
     // ---- SwiGLU * route weight, act_quant per 32 features (this wave's 16 and its neighbour's), 128 code bytes + 4 scales per row
+    unsigned char (*hbuf)[GT_FEAT + 16] = (unsigned char (*)[GT_FEAT + 16])gsm;     // the staging buffers are free: the loop ended on a barrier
     float yv[2][4];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
@@ -757,6 +782,7 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
         if (row < it.n) *(uint32_t*)(hs + (int64_t)(it.off + row) * (I >> 5) + (f0 >> 5)) = *(const uint32_t*)hes[row];
     }
 }
+constexpr size_t UP_GEMM_LDS = (size_t)2 * GT_ROWS * GT_XB;
 
 constexpr int GT_COLS = 256;           // output columns of a down-projection block: two 16-column tiles per wave
 template <int LAYOUT, bool GEN>
@@ -974,8 +1000,14 @@ int moe_launch(const uint8_t* xq, const uint8_t* xs, int R, const int64_t* idx, 
             // the plain forms take K in whole 512-wide groups (gate / up: at most sixteen, down: at most four); a ragged last K group or a
             // longer down product runs the general forms (clamped loads, zero codes past the end, the visit order worked out per group)
             const bool genu = H % 512 != 0, gend = I % 512 != 0 || I / 512 > DN_WAVES;
-            if (genu) up_gemm_kernel<LAYOUT, true><<<dim3(I / GT_FEAT, Gm), 512, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
-            else up_gemm_kernel<LAYOUT, false><<<dim3(I / GT_FEAT, Gm), 512, 0, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
+            static bool attr = false;                      // 65 KB of staging a block: beyond the default cap on dynamic LDS
+            if (!attr) {
+                (void)hipFuncSetAttribute((const void*)up_gemm_kernel<LAYOUT, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)UP_GEMM_LDS);
+                (void)hipFuncSetAttribute((const void*)up_gemm_kernel<LAYOUT, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)UP_GEMM_LDS);
+                attr = true;
+            }
+            if (genu) up_gemm_kernel<LAYOUT, true><<<dim3(I / GT_FEAT, Gm), 512, UP_GEMM_LDS, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
+            else up_gemm_kernel<LAYOUT, false><<<dim3(I / GT_FEAT, Gm), 512, UP_GEMM_LDS, st>>>(xq, xs, m1, m3, H, I, TT, G, items, prow, pw, hq, hs);
             const int hn = H / np;
             const int64_t n4 = (int64_t)R * (hn / 4);
             for (int ps = 0; ps < np; ++ps) {
@@ -1125,6 +1157,18 @@ SPARK_API int spark_mxfp4_moe_x(const void* x, const void* xs, int R, const int6
     }
     if (!mx_fused_ok(R, H, I, topk, E, n_shared)) return 1;
     return mx_fused_launch(x, xs, R, idx, rw, w1, s1, w3, s3, w2, s2, layout, H, I, topk, E, n_shared, add, y, fused_ws(ws, R, H, I, topk, E, n_shared), flags & 1, st, obf16);
+}
+
+// diagnostics: where the several-kernel path (flags bit 1 of spark_mxfp4_moe_x, and every call of more than 8 rows) left the
+// act-quantised intermediate of its last call in a spark_mxfp4_moe* workspace: codes hq [P, I] and scale bytes hs [P, I / 32] in
+// grouped order, prow [P] = the pair (row * (topk + n_shared) + slot) of each grouped row.  Tests compare them with the oracle's.
+SPARK_API int spark_debug_mx_ws_h(void* ws, int R, int H, int I, int topk, int E, int n_shared, void** hq, void** hs, int** prow)
+{
+    if (!shapes_ok(R, H, I, topk, E, n_shared)) return 1;
+    const WsLayout l = ws_layout(R, H, I, topk + n_shared, E + n_shared);
+    char* base = (char*)ws + fused_cap(H, I, topk, E, n_shared);
+    *hq = base + l.hq; *hs = base + l.hs; *prow = (int*)(base + l.prow);
+    return 0;
 }
 
 // ================================================================ C ABI: the reference's symbols (hidden size 5120)

@@ -1,4 +1,5 @@
-// Shared pieces of the MXFP4 expert kernels: weight layouts, the A / B operand loads and the block-scaled MFMA step.
+// Shared pieces of the MXFP4 expert kernels: weight layouts, the A / B operand loads, the exact gate / up step on the bf16 MFMA and
+// the block-scaled MFMA step of the down product.
 //
 // Operand layout of v_mfma_scale_f32_16x16x128_f8f6f4 measured on gfx950: A/B lane l = row/column l % 16, K group g = l / 16.
 // An E2M1 operand holds k = 32 g + e (nibble e of its 16 bytes); an E4M3 operand holds k = 16 g + e in registers 0-3 and
@@ -182,6 +183,59 @@ __device__ __forceinline__ void load_b(const uint8_t* __restrict__ q, const uint
     const uint4 hi = *(const uint4*)(q + step * 128 + 64 + 16 * g);
     b = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
     sb = qs[step * 4 + g];
+}
+
+// ---- gate / up products, exact.  The block-scaled instruction below aligns the products of a 32-block to the block's largest and
+// drops what lies more than about 14 bits under it; the activation quantiser behind the gate / up sums turns some of those 1e-5
+// differences into a flipped E4M3 step of the intermediate.  The reference forms these products exactly (engine-rs/shim/
+// ds41_moe.cu:8-10: E2M1 through a table into bf16, bf16 MMA, binary32 sums), so gate / up run on v_mfma_f32_16x16x32_bf16:
+// E2M1 x 2^sw and E4M3 x 2^sx convert to bf16 exactly (scales inside the hardware convert), every product is exact in
+// binary32 and the sums are binary32.  A 128-wide step is four instructions; instruction j takes, in lane group g, the k
+// 32 g + 8 j .. + 7 of the step from both operands (the contraction index may be dealt to the instructions in any order as long as
+// both operands agree), i.e. dword j of the lane's 16 code bytes as they are streamed: no data crosses lanes.
+typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
+struct XOp { bf8v b[4]; };             // the B operands of a step's four instructions
+// E4M3 bytes lo / hi = k 32 g .. + 15 / + 16 .. + 31 of the step for this lane's token row, sb = the block's UE8M0 byte
+__device__ __forceinline__ XOp x_operand(const uint4& lo, const uint4& hi, uint32_t sb)
+{
+    const float sc = e8m0_to_f32(sb & 0xffu);
+    const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    XOp r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        bf2 v[4];
+        v[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j], sc, false); v[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j], sc, true);
+        v[2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j + 1], sc, false); v[3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j + 1], sc, true);
+        __builtin_memcpy(&r.b[j], v, 16);
+    }
+    return r;
+}
+// row q (E4M3, row stride K) + its UE8M0 scales qs (row stride K / 32): the lane's 32 bytes of the step are neighbours
+__device__ __forceinline__ XOp load_x(const uint8_t* __restrict__ q, const uint8_t* __restrict__ qs, int step, int lane)
+{
+    const int g = lane >> 4;
+    const uint4 lo = *(const uint4*)(q + step * 128 + 32 * g), hi = *(const uint4*)(q + step * 128 + 32 * g + 16);
+    return x_operand(lo, hi, qs[step * 4 + g]);
+}
+// eight E2M1 codes (one dword of the stream, low nibble first) x the block's scale -> the A operand of one instruction
+__device__ __forceinline__ bf8v a_operand(uint32_t w, float sc)
+{
+    bf2 v[4];
+    v[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 0); v[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 1);
+    v[2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 2); v[3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 3);
+    bf8v av;
+    __builtin_memcpy(&av, v, 16);
+    return av;
+}
+// a: the lane's 16 code bytes of step s (block g of 16 weight rows), sa4 byte s: that block's E8M0 scale
+__device__ __forceinline__ v4f mfma_exact_step(int s, const v4i& a, const XOp& x, v4f acc, uint32_t sa4)
+{
+    const float sc = e8m0_to_f32((sa4 >> (8 * s)) & 0xffu);
+    const uint32_t w[4] = {(uint32_t)a.x, (uint32_t)a.y, (uint32_t)a.z, (uint32_t)a.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_operand(w[j], sc), x.b[j], acc, 0, 0, 0);
+    return acc;
 }
 
 template <int OPSEL>

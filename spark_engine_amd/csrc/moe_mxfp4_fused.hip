@@ -5,7 +5,7 @@
 // grouping, combine) than the batch-1 weight stream takes.  Here one grid holds both weight streams:
 //   U blocks: (item, 32 features of I).  8 waves split K as in up_kernel (same summation order, so the values are the
 //       same bits): each wave quantises its K groups of the token rows itself (act_quant per 32, into LDS), streams the 32
-//       gate and 32 up rows, block-scaled MFMA, LDS reduction in wave order, SwiGLU * route weight, act_quant of the 32
+//       gate and 32 up rows, exact products on the bf16 MFMA, LDS reduction in wave order, SwiGLU * route weight, act_quant of the 32
 //       features; the 32 code bytes + scale of every item row go to every stage-2 column block's own copy of h.
 //   D blocks: (64 output columns | item).  Stream their down-projection rows into registers first (raw MXFP4 is the MFMA
 //       operand, nothing to decode), then take the item's h, MFMA as in down_kernel (same order), hand the per-pair
@@ -39,6 +39,7 @@ constexpr int NXCD = 8, HEAD = 256, SPIN_MAX = 200000;
 constexpr uint32_t EMPTY = 0xffffffffu;
 constexpr uint64_t EMPTY2 = ~0ull;
 constexpr int RED_BYTES = NW * 4 * 4 * 64 * 4;
+constexpr size_t XBF_BYTES = 44 * 1024;                   // most bytes of activation rows staged as bf16 (four rows of hidden width 5120)
 
 long long* g_trace = nullptr;
 #ifdef SPK_MX_TRACE
@@ -210,10 +211,9 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
                 for (int s = 0; s < 4; ++s) {
                     const int step = kg * 4 + s;
                     if (step >= steps) break;
-                    v8i b; uint32_t sb;
-                    load_b(xr, xsr, step, lane, b, sb);
+                    const XOp xo = load_x(xr, xsr, step, lane);
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) acc[t] = mfma_group_step(s, A[t][s], b, acc[t], sa[t], sb);
+                    for (int t = 0; t < 4; ++t) acc[t] = mfma_exact_step(s, A[t][s], xo, acc[t], sa[t]);
                 }
             }
 #pragma unroll
@@ -236,21 +236,79 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
             grp_load<LAYOUT>(m, grp.e, row0, q + 2, lane, A[1], sa[1]);
             grp_load<LAYOUT>(m, grp.e, row0, q + 4, lane, A[2], sa[2]);
             grp_load<LAYOUT>(m, grp.e, row0, q + 6, lane, A[3], sa[3]);
-            stage_x(std::integral_constant<bool, !QUANT>{});
+            // Here a wave multiplies one tile with four or five K groups, so converting its activations itself would cost as many
+            // converts again as its weights do: where the rows fit, the block stages them as finished bf16 operands (thread = one
+            // 32-block of a row: act_quant or the caller's codes, then code x 2^scale), else as codes.  The same values either way.
+            const bool xbf = (size_t)a.R * (2 * H + 16) <= XBF_BYTES;
+            const int xbs = 2 * H + 16;                    // row stride of the bf16 rows
+            if (xbf) {
+                // thread = half a 32-block (16 values: few registers beside the weight rows in flight), the two halves are lane neighbours
+                const int nh = H >> 4;
+                for (int u0 = 0; u0 < grp.n * nh; u0 += NT) {
+                    const bool live = u0 + tid < grp.n * nh;                   // the last round's spare threads load the last piece again and store nothing
+                    const int u = live ? u0 + tid : grp.n * nh - 1;
+                    const int r = u / nh, hb = u - r * nh, tok = rows[r] / a.TT;
+                    uint4 cw;
+                    uint32_t sb;
+                    if constexpr (!QUANT) {
+                        cw = *(const uint4*)((const uint8_t*)a.x + (int64_t)tok * H + hb * 16);
+                        sb = a.xs[(int64_t)tok * (H >> 5) + (hb >> 1)];
+                    } else {
+                        const uint4* px = (const uint4*)((const uint16_t*)a.x + (int64_t)tok * H + hb * 16);
+                        const uint4 r0 = px[0], r1 = px[1];
+                        auto lo16 = [](uint32_t w) { return __uint_as_float(w << 16); };
+                        auto hi16 = [](uint32_t w) { return __uint_as_float(w & 0xffff0000u); };
+                        auto amax8 = [&](const uint4& q4) {
+                            return fmaxf(fmaxf(fmaxf(fabsf(lo16(q4.x)), fabsf(hi16(q4.x))), fmaxf(fabsf(lo16(q4.y)), fabsf(hi16(q4.y)))),
+                                         fmaxf(fmaxf(fabsf(lo16(q4.z)), fabsf(hi16(q4.z))), fmaxf(fabsf(lo16(q4.w)), fabsf(hi16(q4.w)))));
+                        };
+                        float am = fmaxf(amax8(r0), amax8(r1));
+                        am = fmaxf(am, lane_xor<1>(am, lane));
+                        sb = aq_scale(am);
+                        cw = make_uint4(aq_word4(lo16(r0.x), hi16(r0.x), lo16(r0.y), hi16(r0.y), sb), aq_word4(lo16(r0.z), hi16(r0.z), lo16(r0.w), hi16(r0.w), sb),
+                                        aq_word4(lo16(r1.x), hi16(r1.x), lo16(r1.y), hi16(r1.y), sb), aq_word4(lo16(r1.z), hi16(r1.z), lo16(r1.w), hi16(r1.w), sb));
+                    }
+                    const float sc = e8m0_to_f32(sb & 0xffu);
+                    const uint32_t w[4] = {cw.x, cw.y, cw.z, cw.w};
+                    unsigned char* d = extra + (size_t)r * xbs + hb * 32;
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        bf2 v[4];
+                        v[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j], sc, false); v[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j], sc, true);
+                        v[2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j + 1], sc, false); v[3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j + 1], sc, true);
+                        uint4 w4; __builtin_memcpy(&w4, v, 16);
+                        if (live) *(uint4*)(d + 16 * j) = w4;
+                    }
+                }
+            } else stage_x(std::integral_constant<bool, !QUANT>{});
             __syncthreads();                               // a wave multiplies K groups that other waves staged
             TRACE(2);
             const uint8_t* xr = xql + (size_t)rc * H;
             const uint8_t* xsr = xsl + (size_t)rc * (H >> 5);
+            const unsigned char* xb = extra + (size_t)rc * xbs + 64 * rg;
             auto unit = [&](v4i (&Au)[4], const GrpScale& sru, int kg, v4f acc) {
                 uint32_t sau;
                 grp_fix<LAYOUT>(Au, sru, lane, sau);
+                if (xbf) {
 #pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const int step = kg * 4 + s;
-                    if (step >= steps) break;
-                    v8i b; uint32_t sb;
-                    load_b(xr, xsr, step, lane, b, sb);
-                    acc = mfma_group_step(s, Au[s], b, acc, sau, sb);
+                    for (int s = 0; s < 4; ++s) {
+                        const int step = kg * 4 + s;
+                        if (step >= steps) break;
+                        const float sc = e8m0_to_f32((sau >> (8 * s)) & 0xffu);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            bf8v b;
+                            { const uint4 w4 = *(const uint4*)(xb + step * 256 + 16 * j); __builtin_memcpy(&b, &w4, 16); }
+                            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_operand((uint32_t)Au[s][j], sc), b, acc, 0, 0, 0);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const int step = kg * 4 + s;
+                        if (step >= steps) break;
+                        acc = mfma_exact_step(s, Au[s], load_x(xr, xsr, step, lane), acc, sau);
+                    }
                 }
                 return acc;
             };
@@ -507,7 +565,8 @@ FPlan fplan(int R, int H, int I, int topk, int E, int n_shared)
     p.hsw = take((size_t)p.NBD * p.P * (I / 32) * 4);
     p.yd = take((size_t)p.P * H * 4);
     p.total = o;
-    const size_t lu = (size_t)R * H + (size_t)R * (H / 32), ld = (size_t)16 * 4 * RMAX * 9 * 4;
+    const size_t xb = (size_t)R * (2 * H + 16);           // nine or ten K groups: the rows as bf16 where they fit
+    const size_t lu = ((H + 511) / 512 > NW && (H + 511) / 512 <= NW + 2 && xb <= XBF_BYTES) ? xb : (size_t)R * H + (size_t)R * (H / 32), ld = (size_t)16 * 4 * RMAX * 9 * 4;
     p.lds = RED_BYTES + ((lu > ld ? lu : ld) + 15) / 16 * 16;
     return p;
 }

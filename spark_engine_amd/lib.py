@@ -86,6 +86,7 @@ SIGNATURES = {
     "spark_moe_ws_status": (i32, [vp, vp]),
     "spark_moe_ws_release": (None, [vp]),
     # diagnostics
+    "spark_debug_mx_ws_h": (i32, [vp, i32, i32, i32, i32, i32, i32, vp, vp, vp]),
     "spark_debug_exl3_local": (None, [i32]), "spark_debug_mx_local": (None, [i32]), "spark_debug_exl3_twa": (None, [i32]),
     "spark_debug_mx_out_cap": (None, [sz]), "spark_debug_validate_routes": (None, [i32]), "spark_mxfp4_moe_path": (i32, [i32] * 7), "spark_exl3_moe_path": (i32, [i32] * 6), "spark_debug_mx_fused_rows": (None, [i32]), "spark_debug_placement": (i32, []), "spark_debug_gemv_rows": (None, [i32]), "spark_debug_fp8q_rowmajor": (None, [i32]),
 }

@@ -29,22 +29,162 @@ def _stacked_mxfp4(ET, H, I, seed):
     return out
 
 
-@pytest.mark.parametrize("R", [1, 2, 4])
-def test_c3_layer_full_shape_vs_oracle(ops, oracle, R):
-    # hidden 4096, intermediate 2048, top-6 + 1 shared, the full expert shape; 24 + 1 experts keep the host side small
-    H, I, E, topk, ns = 4096, 2048, 24, 6, 1
+def _used_experts(t, idx, E, ns=0):
+    """a call whose expert set lives on the device: only the experts its routes name (and the shared ones, which follow the E routed
+    ones) go to the host, renumbered in ascending order -> (host arrays, renumbered routes)"""
+    used = sorted(set(idx.ravel().tolist()))
+    remap = np.full(E, -1, np.int64)
+    remap[used] = np.arange(len(used))
+    sel = torch.tensor(used + list(range(E, E + ns)), device=DEV)
+    return [host(a[sel]) for a in t], remap[idx]
+
+
+def _oracle_on_used_experts(oracle, t, x, idx, rw, E, ns=0, add=None):
+    sub, idx2 = _used_experts(t, idx, E, ns)
+    return oracle.mxfp4_moe(x, idx2, rw, *sub, n_shared=ns, add=add)
+
+
+TIGHT = 1e-4       # where no rounding of the intermediate differs: the down product (block-scaled instruction, 1e-5) and binary32 sums
+NEAR_TIE = 2e-6    # a rounding may come out differently only where the rounded value lies this close to the rounding boundary (sums: relative to the norm of their terms)
+
+
+def _check_against_oracle(oracle, y, gq, gs, prow, t, x, idx, rw, E, topk, ns):
+    """One call (R rows) of the layer held against the oracle THROUGH its intermediate.  The gate / up sums feed three roundings to bf16
+    and a quantiser; two correct evaluations (another order of the binary32 sums, another library's expf) disagree on a rounding
+    only where the rounded value lies on a rounding boundary to within their last places, and then by one step of that element.
+    So: (1) the kernel's act-quantised intermediate (codes gq, scale bytes gs, grouped rows prow) equals the oracle's except in
+    32-blocks that hold an element whose margin (the oracle's own, from binary64 sums) is below NEAR_TIE; (2) the output equals the
+    oracle's down products + sum of the KERNEL's intermediate to TIGHT - which, where (1) found no difference, is the oracle itself.
+    Returns (rel-L2 against the plain oracle per row, number of blocks that differ)."""
+    R, H = x.shape
+    TT, I = topk + ns, gq.shape[1]
+    sub, idx2 = _used_experts(t, idx, E, ns)
+    ref, oq, osb, om = oracle.mxfp4_moe(x, idx2, rw, *sub, n_shared=ns, want_h=True)
+    # the kernel's grouped row g holds pair prow[g] = (row, slot); the oracle lists the routed pairs first, then the shared ones
+    r, k = prow // TT, prow % TT
+    o_of = np.where(k < topk, r * topk + k, R * topk + r * ns + (k - topk))
+    kq, ks = np.empty_like(oq), np.empty_like(osb)
+    kq[o_of], ks[o_of] = gq, gs
+    diff = (kq != oq).reshape(-1, I // 32, 32).any(-1) | (ks != osb)
+    for q, blk in zip(*np.nonzero(diff)):
+        assert om[q, 32 * blk:32 * blk + 32].min() < NEAR_TIE, (int(q), int(blk), float(om[q, 32 * blk:32 * blk + 32].min()))
+    assert diff.sum() <= 4 * R, int(diff.sum())
+    mine = oracle.mxfp4_moe_from_h(kq, ks, idx2, sub[4], sub[5], n_shared=ns) if diff.any() else ref
+    for i in range(R):
+        assert rel_l2(y[i:i + 1], mine[i:i + 1]) <= TIGHT, (i, rel_l2(y[i:i + 1], mine[i:i + 1]))
+    return [rel_l2(y[i:i + 1], ref[i:i + 1]) for i in range(R)], int(diff.sum())
+
+
+def _kernel_intermediate(ops, ws, R, H, I, topk, E, ns):
+    """the act-quantised intermediate the several-kernel path left in ws -> codes [P, I], scale bytes [P, I / 32], prow [P]"""
+    import ctypes as C
+    P = R * (topk + ns)
+    ph, ps, pr = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert ops._lib().spark_debug_mx_ws_h(C.c_void_p(ws.data_ptr()), R, H, I, topk, E, ns, C.byref(ph), C.byref(ps), C.byref(pr)) == 0
+    torch.cuda.synchronize()
+    o = ws.data_ptr()
+    return (ws[ph.value - o:ph.value - o + P * I].view(P, I).cpu().numpy(), ws[ps.value - o:ps.value - o + P * I // 32].view(P, I // 32).cpu().numpy(),
+            ws[pr.value - o:pr.value - o + 4 * P].view(torch.int32).cpu().numpy())
+
+
+@pytest.fixture(scope="module")
+def c3_experts(ops):
+    # config 3 as it is: hidden 4096, intermediate 2048, all 384 routed experts + 1 shared expert on the device
+    H, I, E, ns = 4096, 2048, 384, 1
     t = _stacked_mxfp4(E + ns, H, I, 31)
-    ex = ops.Mxfp4Experts(*t, n_shared=ns)
+    return t, ops.Mxfp4Experts(*t, n_shared=ns)
+
+
+def _c3_call(ops, oracle, t, ex, ws, x, idx, rw):
+    """the single launch, the several-kernel path (the same bits, and its intermediate stays in the workspace), the check"""
+    H, I, E, topk, ns = 4096, 2048, 384, 6, 1
+    R = x.shape[0]
+    xd, idxd, rwd = dev_bf16(x), dev(idx), dev(rw)
+    y = host(ops.mxfp4_moe_x(xd, idxd, rwd, ex, ws=ws, ws_clean=True))
+    xq, xs = ops.act_quant_fp8(xd)
+    y2 = host(ops.mxfp4_moe_x(xq, idxd, rwd, ex, xs=xs, ws=ws, multi_kernel=True))
+    assert np.array_equal(y, y2)
+    gq, gs, prow = _kernel_intermediate(ops, ws, R, H, I, topk, E, ns)
+    return y, _check_against_oracle(oracle, y, gq, gs, prow, t, x, idx, rw, E, topk, ns)
+
+
+@pytest.mark.parametrize("R", [1, 2, 4])
+def test_c3_layer_full_shape_vs_oracle(ops, oracle, c3_experts, R):
+    H, E, topk = 4096, 384, 6
+    t, ex = c3_experts
     g = synth.rng(600 + R)
     x = synth.randn_bf16(g, (R, H))
     logits = g.standard_normal((R, E)).astype(np.float32)
     idx, rw = oracle.ds41_route(logits, np.zeros(E, np.float32), topk, 1.5)
     ws = ops.mxfp4_moe_ws_alloc(R, ex, topk)                  # prepared once: the call is the one launch the benchmark times
-    y = host(ops.mxfp4_moe_x(dev_bf16(x), dev(idx), dev(rw), ex, ws=ws, ws_clean=True))
-    ref = oracle.mxfp4_moe(x, idx, rw, *[host(a) for a in t], n_shared=ns)
-    assert rel_l2(y, ref) <= TOL, rel_l2(y, ref)
+    y, (errs, _) = _c3_call(ops, oracle, t, ex, ws, x, idx, rw)
+    assert max(errs) <= TOL, errs
     assert np.array_equal(host(ops.mxfp4_moe_x(dev_bf16(x), dev(idx), dev(rw), ex, ws=ws, ws_clean=True)), y)
     ops.ws_check(ws)
+
+
+NROWS = 256
+
+
+def _report(name, errs, nd):
+    errs = np.array(errs)
+    print(f"{name}: {len(errs)} token rows sent alone: rel-L2 against the oracle median {np.median(errs):.2e}, worst {errs.max():.2e}; "
+          f"{int((np.array(nd) > 0).sum())} rows with a rounding of the intermediate on a near-tie ({int(np.sum(nd))} blocks), "
+          f"{int((errs > TOL).sum())} of them beyond {TOL:g}")
+    # rows without such a rounding sit at the down product's 1e-5; one flipped E4M3 step of a large element costs up to a few 1e-3
+    assert (errs[np.array(nd) == 0] <= TIGHT).all() and errs.max() <= 5e-3 and (errs > TOL).mean() <= 0.02
+
+
+def test_c3_every_token_row_sent_alone(ops, oracle, c3_experts):
+    # A batch-1 decode call is one token row, so the reference's bar for the layer (rel-L2 < 1e-3 against moe_ref,
+    # engine-rs/src/ds41/kern.rs:2206-2208, a single random row there) is looked at row by row: every row must match the oracle
+    # through its intermediate (_check_against_oracle), which is far tighter than 1e-3 wherever no rounding sits on a tie.
+    H, E, topk = 4096, 384, 6
+    t, ex = c3_experts
+    g = synth.rng(640)
+    x = synth.randn_bf16(g, (NROWS, H))
+    logits = g.standard_normal((NROWS, E)).astype(np.float32)
+    idx, rw = oracle.ds41_route(logits, np.zeros(E, np.float32), topk, 1.5)
+    ws = ops.mxfp4_moe_ws_alloc(1, ex, topk)
+    errs, nd = [], []
+    for r in range(NROWS):
+        _, (e, n) = _c3_call(ops, oracle, t, ex, ws, x[r:r + 1], idx[r:r + 1], rw[r:r + 1])
+        errs += e; nd.append(n)
+    ops.ws_check(ws)
+    _report("C3", errs, nd)
+
+
+@pytest.mark.parametrize("I", [768, 2048])
+def test_ds41_moe_mx_every_token_row_sent_alone(ops, oracle, I):
+    # the same through the reference's own entry point and tile layout (hidden 5120; 768 = the reference's intermediate width per
+    # rank of three, engine-rs/src/ds41/kern.rs:2179-2190), 384 experts top-6
+    import ctypes as C
+    H, E, topk = 5120, 384, 6
+    t = _stacked_mxfp4(E, H, I, 34)
+    p1, ps1 = ops.moe_pack(t[0], t[1]); p3, ps3 = ops.moe_pack(t[2], t[3]); p2, ps2 = ops.moe_pack(t[4], t[5])
+    w = (ops.moe_pack_mx(p1), ps1, ops.moe_pack_mx(p3), ps3, ops.moe_pack_mx(p2), ps2)
+    del p1, p3, p2
+    g = synth.rng(641 + I)
+    x = synth.randn_bf16(g, (NROWS, H))
+    logits = g.standard_normal((NROWS, E)).astype(np.float32)
+    idx, rw = oracle.ds41_route(logits, np.zeros(E, np.float32), topk, 1.5)
+    xq, xs = ops.act_quant_fp8(dev_bf16(x))
+    idxd, rwd = dev(idx), dev(rw)
+    L = ops._lib()
+    wsb = torch.empty(L.ds41_moe_mx_ws_bytes(1, I, topk, E), dtype=torch.uint8, device=DEV)
+    y2 = torch.empty(1, H, dtype=torch.float32, device=DEV)
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    errs, nd = [], []
+    for r in range(NROWS):
+        y, _ = ops.ds41_moe_mx(xq[r:r + 1], xs[r:r + 1], idxd[r:r + 1], rwd[r:r + 1], w, I, ws=wsb)          # one launch
+        y = host(y)
+        ops.ds41_moe_mx(xq[r:r + 1], xs[r:r + 1], idxd[r:r + 1], rwd[r:r + 1], w, I, ws=wsb, skip_combine=True)   # the several-kernel path ...
+        assert L.ds41_moe_mx_combine(C.c_void_p(wsb.data_ptr()), 1, I, topk, E, None, C.c_void_p(y2.data_ptr()), st) == 0
+        assert np.array_equal(host(y2), y)                                                                # ... gives the same bits
+        gq, gs, prow = _kernel_intermediate(ops, wsb, 1, H, I, topk, E, 0)
+        e, n = _check_against_oracle(oracle, y, gq, gs, prow, t, x[r:r + 1], idx[r:r + 1], rw[r:r + 1], E, topk, 0)
+        errs += e; nd.append(n)
+    _report(f"ds41_moe_mx I {I}", errs, nd)
 
 
 @pytest.mark.parametrize("N,K", [(7168, 4096), (4096, 7168)])
@@ -97,12 +237,13 @@ def test_c5_prefill_rows_equal_decode_rows(ops, oracle):
     for r in rows:                                                       # the same row alone, through the single-launch decode path
         one = host(ops.mxfp4_moe_x(xd[r:r + 1], idxd[r:r + 1], rwd[r:r + 1], ex))
         assert np.array_equal(one[0], yh[r]), r
-    for r in rows[:2]:                                                   # and against the oracle (only the row's experts go to the host)
-        used = sorted(set(idx[r].tolist()))
-        remap = {e: i for i, e in enumerate(used)}
-        sub = [host(a[used]) for a in t]
-        ref = oracle.mxfp4_moe(x[r:r + 1], np.array([[remap[e] for e in idx[r]]], np.int64), rw[r:r + 1], *sub)
-        assert rel_l2(yh[r:r + 1], ref) <= TOL
+    errs = []
+    for r in rows + list(range(3, R, 64)):                               # and every 64th row against the oracle (only a row's experts go to the host)
+        errs.append(rel_l2(yh[r:r + 1], _oracle_on_used_experts(oracle, t, x[r:r + 1], idx[r:r + 1], rw[r:r + 1], E)))
+    print(f"C5 rows: worst rel-L2 {max(errs):.3e}, median {np.median(errs):.3e}")
+    # a row whose intermediate has a rounding on a near-tie can exceed the bar (test_c3_every_token_row_sent_alone); the rows of a
+    # prefill call are the decode rows bit for bit, so that is checked there: here the sample's bulk and the worst case
+    assert np.median(errs) <= TIGHT and max(errs) <= 5e-3, max(errs)
 
 
 def test_c2_layer_rows_do_not_depend_on_the_batch(ops, oracle):

@@ -99,39 +99,68 @@ def test_exl3_moe_weighted_sum_add_and_row_invariance(oracle):
     assert np.array_equal(oracle.exl3_moe(x[1:2], idx[1:2], w[1:2], experts, E, H, I, 4, 2, 0, add[1:2])[0], out[1])
 
 
-def _ds41_pair_torch(xd, w1, s1, w3, s3, w2, s2, rw, oracle):
-    """reference ds41/kern.rs:1116-1133 (moe_ref) for one pair, with torch ops."""
-    bf = lambda t: t.to(torch.bfloat16).float()
-    deq = lambda w, s: torch.from_numpy(oracle.mxfp4_dequant(w, s))
-    x = torch.from_numpy(xd)[None]
-    g = bf(x @ deq(w1, s1).T).clamp_max(10.0)
-    u = bf(x @ deq(w3, s3).T).clamp(-10.0, 10.0)
-    hm = (F.silu(g) * u * rw).to(torch.bfloat16)
-    hb = hm.view(torch.int16).numpy().view(np.uint16)
-    hq = torch.from_numpy(oracle.bf16_to_f32(oracle.act_quant32(hb)))
-    return (hq @ deq(w2, s2).T)[0].numpy()
+def _ds41_pair_stages(xd, w1, s1, w3, s3, w2, s2, rw, oracle):
+    """reference ds41/kern.rs:1116-1133 (moe_ref) for one pair, stage by stage with library routines: the gate / up sums in
+    binary64 (exact for these terms, whatever the order), the activation in binary64 too, the quantiser through
+    torch.float8_e4m3fn.  -> E4M3 codes [I], scale bytes [I / 32], and which 32-blocks are robust: no element's product within 1e-6
+    of a bf16 rounding boundary, so that a last-place difference of expf cannot change a code or the block's scale."""
+    from tests.gpu_util import bf16_safe
+    bf = lambda t: t.float().to(torch.bfloat16).double()
+    deq = lambda w, s: torch.from_numpy(oracle.mxfp4_dequant(w, s)).double()
+    x = torch.from_numpy(xd).double()[None]
+    g = bf(x @ deq(w1, s1).T).clamp_max(10.0)[0]
+    u = bf(x @ deq(w3, s3).T).clamp(-10.0, 10.0)[0]
+    y64 = g / (1.0 + torch.exp(-g)) * u * float(np.float32(rw))
+    # element by element: none of its three roundings within 1e-6 of a rounding boundary (gate / up sums: of the norm of their terms; product: of itself)
+    tnorm = lambda w, s: torch.sqrt((x * x) @ (deq(w, s) ** 2).T)[0].numpy()                       # the norm of each sum's terms
+    esafe = (bf16_safe(y64.numpy(), margin=1e-6) & bf16_safe((x @ deq(w1, s1).T)[0].numpy(), margin=1e-6, size=tnorm(w1, s1)) &
+             bf16_safe((x @ deq(w3, s3).T)[0].numpy(), margin=1e-6, size=tnorm(w3, s3)))
+    safe = torch.from_numpy(bf16_safe(y64.numpy(), margin=1e-6)).view(-1, 32).all(dim=1).numpy()
+    yb = y64.float().to(torch.bfloat16).float().view(-1, 32)
+    amax = yb.abs().amax(dim=1).clamp_min(1e-4)
+    e = torch.ceil(torch.log2(amax.double() / 448.0)).to(torch.int32)              # scale = 2^ceil(log2(amax / 448)), reference kernel.py:59-73
+    q = (yb.double() / torch.pow(2.0, e.double())[:, None]).clamp(-448.0, 448.0).float().to(torch.float8_e4m3fn)
+    return q.view(torch.uint8).view(-1).numpy(), (e + 127).to(torch.uint8).numpy(), safe, esafe
 
 
-def test_mxfp4_moe_vs_torch_restatement(oracle):
+def test_mxfp4_moe_stage_by_stage_vs_library_routines(oracle):
     g = synth.rng(5)
-    H, I, E, topk, R = 256, 128, 5, 2, 3
+    H, I, E, topk, R = 512, 256, 5, 2, 3
     ws = synth.mxfp4_experts(g, E + 1, H, I, smin=119)
     x = synth.randn_bf16(g, (R, H))
     idx = np.array([[0, 3], [3, 4], [1, 2]], np.int64)
     rw = g.uniform(0.2, 1.0, (R, topk)).astype(np.float32)
     add = g.standard_normal((R, H)).astype(np.float32)
-    y, pairs = oracle.mxfp4_moe(x, idx, rw, *ws, n_shared=1, add=add, want_pairs=True)
+    y, pairs, hq, hs, hmargin = oracle.mxfp4_moe(x, idx, rw, *ws, n_shared=1, add=add, want_pairs=True, want_h=True)
     xd = oracle.bf16_to_f32(oracle.act_quant32(x))
-    for r in range(R):
-        acc = np.zeros(H, np.float32)
-        for k in range(topk):
-            e = int(idx[r, k])
-            ref = _ds41_pair_torch(xd[r], ws[0][e], ws[1][e], ws[2][e], ws[3][e], ws[4][e], ws[5][e], float(rw[r, k]), oracle)
-            assert np.linalg.norm(pairs[r * topk + k] - ref) <= 2e-3 * np.linalg.norm(ref)   # bf16 / e4m3 roundings may flip on summation order
-            acc = acc + pairs[r * topk + k]
-        sh = _ds41_pair_torch(xd[r], ws[0][E], ws[1][E], ws[2][E], ws[3][E], ws[4][E], ws[5][E], 1.0, oracle)
-        full = add[r] + sh + acc
-        assert np.linalg.norm(y[r] - full) <= 2e-3 * np.linalg.norm(full)
+    P = R * topk
+    nblocks = nsafe = 0
+    for p in range(P + R):                                             # routed pairs, then the shared expert of every row
+        r, e, w = (p // topk, int(idx.ravel()[p]), float(rw.ravel()[p])) if p < P else (p - P, E, 1.0)
+        q, sb, safe, esafe = _ds41_pair_stages(xd[r], *[a[e] for a in ws], w, oracle)
+        # the oracle's own rounding margins say the same, element by element (elements right at the threshold aside)
+        clear = np.abs(hmargin[p] - 1e-6) > 1e-7
+        assert np.array_equal((hmargin[p] > 1e-6)[clear], esafe[clear])
+        nblocks += safe.size; nsafe += int(safe.sum())
+        # the intermediate: codes and scale bytes equal on every robust block (a dropped rounding, a missing route weight, a wrong
+        # clamp or scale rule changes nearly every block)
+        assert np.array_equal(hs[p][safe], sb[safe])
+        assert np.array_equal(hq[p].reshape(-1, 32)[safe], q.reshape(-1, 32)[safe])
+        # the down product of the oracle's own codes, in binary64
+        hm = torch.from_numpy(hq[p].copy()).view(torch.float8_e4m3fn).double() * torch.pow(2.0, torch.from_numpy(hs[p].astype(np.float64)) - 127.0).repeat_interleave(32)
+        out = (hm[None] @ torch.from_numpy(oracle.mxfp4_dequant(ws[4][e], ws[5][e])).double().T)[0].numpy()
+        if p < P:
+            assert np.linalg.norm(pairs[p] - out) <= 1e-5 * np.linalg.norm(out)
+        else:
+            routed = np.zeros(H, np.float32)
+            for k in range(topk):
+                routed = routed + pairs[r * topk + k]                  # slot order, then added to add + shared (reference ds41_mx.cu:302-317)
+            full = (add[r].astype(np.float64) + out) + routed
+            assert np.linalg.norm(y[r] - full) <= 1e-5 * np.linalg.norm(full)
+    assert nsafe >= 0.9 * nblocks, (nsafe, nblocks)                   # the exact comparison covers nearly everything
+    assert (hmargin < 1e-6).sum() >= 1                                # and the margins do flag something at this size
+    # the second half alone, on the oracle's own intermediate, is the whole: same operations in the same order
+    assert np.array_equal(oracle.mxfp4_moe_from_h(hq, hs, idx, ws[4], ws[5], n_shared=1, add=add), y)
     # zero codes -> zero expert output: y == add
     zw = [np.zeros_like(a) if i % 2 == 0 else a for i, a in enumerate(ws)]
     y0 = oracle.mxfp4_moe(x, idx, rw, *zw, n_shared=1, add=add)
