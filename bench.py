@@ -45,7 +45,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--batch", type=int, default=1, help="tokens per step of the headline workload (1 or 4)")
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c2q", "c2g", "c2ref", "c2refp", "c3", "c3w", "c3ref", "c3refp", "c3rank", "c4a", "c4b", "c4ap", "c4bp", "p1", "p2", "p3", "c5", "c5w", "c2p"],
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c2q", "c2g", "c2ref", "c2refp", "c3", "c3w", "c3ref", "c3refp", "c3rank", "c4a", "c4b", "c4ap", "c4bp", "p1", "p2", "p3", "g8", "c5", "c5w", "c2p"],
                     help="headline workload: c2 EXL3 MoE (default, the metric's configuration), c3 MXFP4 MoE (c3w: the same at hidden width 5120), c4a/c4b FP8 dense 7168x4096 / 4096x7168")
     ap.add_argument("--only-headline", action="store_true", help="skip the other configurations' lines")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -510,6 +510,75 @@ class Fp8MxProjection:
         return self.N * self.K + self.s[0].numel() + self.R * (self.K + self.K // 32) + self.R * self.N * 4, 1.0
 
 
+class GlmFp8Dense:
+    """The reference's GLM dense / shared-expert projection format (reference engine-rs/shim/fp8.cu:13-22,110-128): E4M3 weights with one
+    binary32 scale per output row, binary32 activations rounded to binary16 inside (glm53_fp8_dense_cuda).  Not one of the five configurations."""
+    LAYERS = 1
+    DTYPE = "fp8 x f16 (E4M3 weights with a scale per output row, binary16 activations, fp32 accumulate)"
+    SET = "rotating over more than 512 MB of weight copies"
+
+    def __init__(self, torch, ops, R, inst, N, K, seed=8):
+        self.torch, self.ops, self.R, self.inst, self.N, self.K = torch, ops, R, inst, N, K
+        dev = "cuda:0"
+        g = torch.Generator(device=dev).manual_seed(seed)
+        ncopy = max(2, min(inst, (600 << 20) // (N * K) + 1))
+        self.w = torch.randn(ncopy, N, K, device=dev, generator=g).clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+        self.s = torch.rand(ncopy, N, device=dev, generator=g) * 1e-2 + 1e-3
+        self.x = torch.randn(R, K, device=dev, generator=g)
+        self.y = torch.empty(R, N, dtype=torch.float32, device=dev)
+        self.ncopy = ncopy
+        self.name = f"GLM-format FP8 dense GEMV {N}x{K} (one scale per output row, glm53_fp8_dense_cuda), batch {R}"
+
+    def step(self, i):
+        c = i % self.ncopy
+        L, ops = self.ops._lib(), self.ops
+        ops._ck(L.glm53_fp8_dense_cuda(ops._p(self.x), ops._p(self.w[c]), ops._p(self.s[c]), ops._p(self.y), None, self.R, self.N, self.K, 0, 1, 0, ops._st()),
+                "glm53_fp8_dense_cuda")
+
+    def bytes_per_step(self):
+        return self.N * self.K + self.N * 4 + self.R * self.K * 4 + self.R * self.N * 4, 1.0
+
+    def cpu_sample(self, orc, budget_s=4.0):
+        x, w, sc = self.x.cpu().numpy(), self.w[0].cpu().numpy(), self.s[0].cpu().numpy()
+        times = []
+        for _ in range(4):
+            t0 = time.perf_counter()
+            ref = orc.fp8_rowscale_gemv(x, w, sc, act=0)
+            times.append(time.perf_counter() - t0)
+        self.step(0)
+        got = self.y.cpu().numpy()
+        return (float(np.median(times[1:])) * 1e6, "the whole projection (E4M3 decode + dot products in binary64, OpenMP), median of 3 after one warm-up",
+                float(np.linalg.norm(got - ref) / np.linalg.norm(ref)))
+
+
+class StreamFloor:
+    """The stream floor of a line: a plain read (non-temporal 16-byte loads, one small store) of exactly the line's algorithmic bytes,
+    timed in the same graph of instances, each instance on its own region of a buffer larger than the caches."""
+
+    def __init__(self, torch, ops, nbytes, inst):
+        self.torch, self.ops, self.inst = torch, ops, inst
+        self.nbytes = int(nbytes) // 16 * 16
+        span = max(self.nbytes * min(inst, 64), 1 << 30)
+        self.regions = max(1, min(inst, span // self.nbytes))
+        self.buf = torch.empty(self.regions * self.nbytes, dtype=torch.uint8, device="cuda:0")
+        self.buf.view(torch.int32).random_(0, 1 << 30)
+        self.out = torch.zeros(1024, dtype=torch.int32, device="cuda:0")
+
+    def step(self, i):
+        ops = self.ops
+        ops._ck(ops._lib().spark_debug_stream_read(self.buf.data_ptr() + (i % self.regions) * self.nbytes, self.nbytes, ops._p(self.out), ops._st()),
+                "spark_debug_stream_read")
+
+
+def stream_floor(torch, ops, nbytes, inst):
+    """us to read nbytes: median per instance of the timing protocol's graph"""
+    f = StreamFloor(torch, ops, nbytes, inst)
+    us = time_protocol(torch, f, replays=10, warm=3)[0]
+    del f
+    torch.cuda.empty_cache()
+    return us
+
+
 class Mxfp4Dense:
     """Config 1: MXFP4 dense GEMV 2048 x 2048, one row (the reference's own CPU-runnable case, reference ds41.cu:75-110, 236)."""
     LAYERS = 1
@@ -622,7 +691,9 @@ def time_steps(torch, wl, steps, warmup, fn=None):
     return e0.elapsed_time(e1) / steps
 
 
-def line_for(wl, us, lo, hi, lat):
+def line_for(wl, us, lo, hi, lat, tag=None, floor=None):
+    """tag: the line's name in profiles/hbm_counters_*.txt (counter traffic of its dominant kernel or whole call); floor: (torch, ops) to time
+    the stream floor of the line's algorithmic bytes"""
     by, d = wl.bytes_per_step()
     gbs = by / (us * 1e-6) / 1e9
     out = {"workload": wl.name, "us_per_layer": round(us, 3), "us_per_layer_min_max": [round(lo, 3), round(hi, 3)], "single_call_latency_us": round(lat, 2),
@@ -634,6 +705,12 @@ def line_for(wl, us, lo, hi, lat):
         peak = getattr(wl, "MFMA_PEAK_TFLOPS", FP8_PEAK_TFLOPS)      # fp16 operands for the EXL3 GEMM, fp8 for the MXFP4 one
         out.update({"flops": wl.flops, "achieved_TFLOPs": round(tf, 1), "mfma_peak_TFLOPs": peak, "frac_of_mfma_peak": round(tf / peak, 4),
                     "time_at_hbm_peak_us": round(by / (HBM_PEAK_GBS * 1e9) * 1e6, 1), "time_at_mfma_peak_us": round(wl.flops / (peak * 1e12) * 1e6, 1)})
+    if tag is not None:
+        out["traffic"], out["traffic_source"] = counter_traffic(tag)
+    if floor is not None:
+        fl = stream_floor(floor[0], floor[1], by, wl.inst)
+        out["stream_floor_us"] = round(fl, 3)
+        out["frac_of_floor"] = round(fl / us, 4)
     return out
 
 
@@ -687,7 +764,7 @@ def main():
         "c5": lambda: Mxfp4Prefill(torch, ops, 2048, 4), "c5w": lambda: Mxfp4PrefillWide(torch, ops, 2048, 4), "c2p": lambda: Exl3Prefill(torch, ops, 2048, 4),
         "c4a": lambda: Fp8Dense(torch, ops, a.batch, INST, 7168, 4096), "c4b": lambda: Fp8Dense(torch, ops, a.batch, INST, 4096, 7168),
         "p1": lambda: Fp8MxProjection(torch, ops, a.batch, INST, 12288, 1280), "p2": lambda: Fp8MxProjection(torch, ops, a.batch, INST, 5120, 3072),
-        "p3": lambda: Fp8MxProjection(torch, ops, a.batch, INST, 1280, 5120),
+        "p3": lambda: Fp8MxProjection(torch, ops, a.batch, INST, 1280, 5120), "g8": lambda: GlmFp8Dense(torch, ops, a.batch, INST, 4096, 4096),
         "c4ap": lambda: Fp8DensePacked(torch, ops, a.batch, INST, 7168, 4096), "c4bp": lambda: Fp8DensePacked(torch, ops, a.batch, INST, 4096, 7168),
     }
     wl = make[a.config]()
@@ -699,7 +776,7 @@ def main():
     ms = time_steps(torch, wl, a.steps, a.warmup)
     us, lo, hi, lat = time_protocol(torch, wl)
     check_ws(ops, wl)
-    head = line_for(wl, us, lo, hi, lat)
+    head = line_for(wl, us, lo, hi, lat, tag=f"{a.config} batch{wl.R}", floor=(torch, ops))
     # the dominant kernel alone, same graph and events: its average launch duration prices the roofline
     if getattr(wl, "dominant", None) is not None:
         k_us = time_protocol(torch, wl, wl.dominant)[0]
@@ -711,28 +788,32 @@ def main():
     cpu = cpu_leg(wl, orc, 12.0) if orc is not None else None
     if cpu is not None:
         head["cpu_baseline"] = cpu
-    traffic, traffic_src = counter_traffic(f"{a.config} batch{wl.R}")
+    traffic, traffic_src = head["traffic"], head["traffic_source"]
     others = []
     if not a.only_headline:
         del wl
         torch.cuda.empty_cache()
-        todo = [lambda: Mxfp4Dense(torch, ops, 1, 256)]                                   # C1 first: it is defined as the CPU path
-        todo += [lambda: Exl3Layer(torch, ops, 4 if a.batch == 1 else 1, INST)]
-        todo += [lambda R=R: Mxfp4Layer(torch, ops, R, INST) for R in (1, 2, 4)]
-        todo += [lambda R=R, N=N, K=K: Fp8Dense(torch, ops, R, INST, N, K) for (N, K) in ((7168, 4096), (4096, 7168)) for R in (1, 4)]
-        todo += [lambda R=R, N=N, K=K: Fp8DensePacked(torch, ops, R, INST, N, K) for (N, K) in ((7168, 4096), (4096, 7168)) for R in (1, 4)]
-        todo += [lambda: Mxfp4Prefill(torch, ops, 2048, 4), lambda: Exl3Prefill(torch, ops, 2048, 4)]
+        # (workload, its tag in profiles/hbm_counters_*.txt or None)
+        todo = [(lambda: Mxfp4Dense(torch, ops, 1, 256), "c1 batch1")]                      # C1 first: it is defined as the CPU path
+        ob = 4 if a.batch == 1 else 1
+        todo += [(lambda: Exl3Layer(torch, ops, ob, INST), f"c2 batch{ob}")]
+        todo += [(lambda R=R: Mxfp4Layer(torch, ops, R, INST), f"c3 batch{R}") for R in (1, 2, 4)]
+        todo += [(lambda R=R, N=N, K=K: Fp8Dense(torch, ops, R, INST, N, K), f"{c} batch{R}") for (c, N, K) in (("c4a", 7168, 4096), ("c4b", 4096, 7168)) for R in (1, 4)]
+        todo += [(lambda R=R, N=N, K=K: Fp8DensePacked(torch, ops, R, INST, N, K), f"{c} batch{R}") for (c, N, K) in (("c4ap", 7168, 4096), ("c4bp", 4096, 7168)) for R in (1, 4)]
+        todo += [(lambda: Mxfp4Prefill(torch, ops, 2048, 4), "c5 batch2048"), (lambda: Exl3Prefill(torch, ops, 2048, 4), "c2p batch2048")]
         # the reference model's dense projections (not a configuration: the callers either side of the expert layer)
-        todo += [lambda N=N, K=K, R=R: Fp8MxProjection(torch, ops, R, INST, N, K) for (N, K) in ((12288, 1280), (5120, 3072), (1280, 5120)) for R in (1, 8)]
+        todo += [(lambda N=N, K=K, R=R: Fp8MxProjection(torch, ops, R, INST, N, K), None) for (N, K) in ((12288, 1280), (5120, 3072), (1280, 5120)) for R in (1, 8)]
+        todo += [(lambda R=R: GlmFp8Dense(torch, ops, R, INST, 4096, 4096), None) for R in (1, 4)]
         # the sizes the reference's own kernels are compiled for, through spark_* and through the reference-named entry points
         # (a caller that changes nothing: workspace contents undefined, no *_ws_init; and with the one added *_ws_init call)
-        todo += [lambda: Exl3LayerQwen(torch, ops, 1, INST), lambda: QwenReferenceEntry(torch, ops, 1, INST, prepared=False),
+        todo += [(mk, None) for mk in (
+                 lambda: Exl3LayerQwen(torch, ops, 1, INST), lambda: QwenReferenceEntry(torch, ops, 1, INST, prepared=False),
                  lambda: QwenReferenceEntry(torch, ops, 1, INST, prepared=True), lambda: Exl3LayerGlm(torch, ops, 1, INST),
                  lambda: Mxfp4LayerWide(torch, ops, 1, INST), lambda: Ds41ReferenceEntry(torch, ops, 1, INST, prepared=False),
-                 lambda: Ds41ReferenceEntry(torch, ops, 1, INST, prepared=True), lambda: Ds41ReferenceEntryRank(torch, ops, 1, INST, prepared=True)]
-        for mk in todo:
+                 lambda: Ds41ReferenceEntry(torch, ops, 1, INST, prepared=True), lambda: Ds41ReferenceEntryRank(torch, ops, 1, INST, prepared=True))]
+        for mk, tag in todo:
             w2 = mk()
-            ln = line_for(w2, *time_protocol(torch, w2))
+            ln = line_for(w2, *time_protocol(torch, w2), tag=tag, floor=(torch, ops))
             check_ws(ops, w2)
             if orc is not None:
                 c2 = cpu_leg(w2, orc, 4.0)
@@ -754,7 +835,9 @@ def main():
                    "tok_per_s_equiv": head["tok_per_s_equiv"], "layers_assumed": head["layers_assumed"]},
         "roofline": {"bound": "hbm", "achieved": round(k_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(k_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "traffic_source": traffic_src, "kernel": k_name, "kernel_us_per_launch": round(k_us, 3), "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
-                     "whole_layer_GBps": head["achieved_GBps"], "whole_layer_frac": head["frac_of_hbm_peak"]},
+                     "whole_layer_GBps": head["achieved_GBps"], "whole_layer_frac": head["frac_of_hbm_peak"],
+                     # a plain read of the launch's algorithmic bytes in the same graph of instances, and the kernel's time against it
+                     "stream_floor_us": head["stream_floor_us"], "frac_of_floor": round(head["stream_floor_us"] / k_us, 4)},
         "cpu_baseline": cpu,
         "all_configs": [head] + others,
     }

@@ -192,6 +192,22 @@ SPARK_API int ds41_moe_mx(const void* xq, const void* xs, int R, const int64_t* 
 SPARK_API int ds41_moe_mx_combine_rows(void* ws, int R, int I, int topk, int E, const float* add, float* y, int r0, int nr, hipStream_t st);
 SPARK_API int ds41_moe_mx_combine(void* ws, int R, int I, int topk, int E, const float* add, float* y, hipStream_t st);
 SPARK_API int ds41_moe_mx_ws_ptrs(void* ws, int R, int I, int topk, int E, float** out, int** pairmap);
+/* Weight-only FP8 with one binary32 scale per output row (the GLM dense / shared-expert projections; quantiser
+ * engine-rs/src/dense_fp8.rs:59-62: scale = row amax / 448):  y[r, n] = (sum_k a(x[r, k]) * e4m3(w[n, k])) * scales[n].
+ * x binary32 [m, k], w E4M3 [n, k], scales binary32 [n], y binary32 [m, n]; exact products, binary32 sums; a row's value does not
+ * depend on the rows beside it.  Return 0, or 1 (the reference's cudaErrorInvalidValue) for a shape outside the stated limits.
+ * glm53_fp8_dense_cuda: a = round to binary16, m 1..16, n and k multiples of 64; rounded != 0: every output rounded to binary16.
+ *   scratch, mode and split_override pick among the reference's kernels and feed its split-K forms: accepted, not used (one kernel
+ *   family here, K split by the shape).  Replaces engine-rs/shim/fp8.cu:110-128.
+ * glm53_fp8_bf16_cuda: a = round to bf16, no output rounding; splits must be 1, 2, 4, 8 or 16 and is otherwise unused.
+ *   Replaces engine-rs/shim/fp8.cu:143-151.
+ * glm53_fp8_bf16_skinny_cuda: bf16 activations read as they are, m 2..32, n a multiple of 16.  Replaces engine-rs/shim/fp8.cu:134-141. */
+SPARK_API int glm53_fp8_dense_cuda(const float* x, const void* w, const float* scales, float* y, float* scratch, int m, int n, int k, int rounded,
+                                   int mode, int split_override, hipStream_t st);
+SPARK_API int glm53_fp8_bf16_cuda(const float* x, const void* w, const float* scales, float* y, float* scratch, int m, int n, int k, int splits,
+                                  hipStream_t st);
+SPARK_API int glm53_fp8_bf16_skinny_cuda(const void* x_bf16, const void* w, const float* scales, float* y, int m, int n, int k, hipStream_t st);
+
 /* bf16 activations (already act-quantised), weights in the moe_pack layout.  Replaces engine-rs/shim/ds41_moe.cu:259-292. */
 SPARK_API size_t ds41_moe_ws_bytes(int R, int I, int topk, int E);
 SPARK_API int ds41_moe(const void* xq, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3,
@@ -310,6 +326,10 @@ SPARK_API void spark_debug_mx_fused_rows(int rows);
  * grouped order, prow [P] = the pair (row * (topk + n_shared) + slot) of each grouped row.  For tests that compare the
  * intermediate with the CPU oracle's; returns 1 on a shape the entry points refuse. */
 SPARK_API int spark_debug_mx_ws_h(void* ws, int R, int H, int I, int topk, int E, int n_shared, void** hq, void** hs, int** prow);
+/* The stream floor: reads `bytes` bytes (rounded down to 16) at src (device memory, 16-byte aligned) with non-temporal 16-byte loads
+ * and stores one word a wave into out (device memory of 4096 bytes): the time it takes bounds from below every kernel that must
+ * fetch that many bytes from memory.  The benchmark times it in the same graph of instances as the layers.  1 = bad arguments. */
+SPARK_API int spark_debug_stream_read(const void* src, size_t bytes, void* out, hipStream_t st);
 /* k-tiles per wave of a stage-1 block of the single-launch EXL3 kernel: 4 or 8 forces it, 0 = chosen by the shape (the default) */
 SPARK_API void spark_debug_exl3_twa(int v);
 

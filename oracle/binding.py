@@ -49,6 +49,8 @@ def _load():
         "orc_mxfp4_gemv": (None, [vp, vp, vp, vp, i32, i32, i32]),
         "orc_fp8_block_gemv": (None, [vp, vp, vp, vp, i32, i32, i32, i32]),
         "orc_fp8_e8m0_gemv": (None, [vp, vp, vp, vp, i32, i32, i32]),
+        "orc_fp8_rowscale_gemv": (None, [vp, vp, vp, vp, i32, i32, i32, i32, i32]),
+        "orc_fp8_rowscale_quant": (None, [vp, vp, vp, i32, i32]),
         "orc_num_threads": (i32, []),
     }
     for name, (res, args) in sig.items():
@@ -314,6 +316,26 @@ def fp8_e8m0_gemv(x_bits, w, s):
     y = np.empty((m, n), np.float32)
     lib.orc_fp8_e8m0_gemv(_p(x_bits), _p(w), _p(s), _p(y), m, n, k)
     return y
+
+
+def fp8_rowscale_gemv(x, w, scale, act=0, rounded=False):
+    """x f32 [m, k] (act 0: rounded to f16, 1: to bf16, 2: as given), w E4M3 [n, k], scale f32 [n] -> y f32 [m, n]."""
+    x, w, scale = _c(x, np.float32), _c(w, np.uint8), _c(scale, np.float32)
+    m, k = x.shape
+    n = w.shape[0]
+    y = np.empty((m, n), np.float32)
+    lib.orc_fp8_rowscale_gemv(_p(x), _p(w), _p(scale), _p(y), m, n, k, act, int(rounded))
+    return y
+
+
+def fp8_rowscale_quant(w):
+    """w f32 [n, k] -> (E4M3 codes [n, k], scales f32 [n]) by the reference's row-amax rule."""
+    w = _c(w, np.float32)
+    n, k = w.shape
+    q = np.empty((n, k), np.uint8)
+    s = np.empty(n, np.float32)
+    lib.orc_fp8_rowscale_quant(_p(w), _p(q), _p(s), n, k)
+    return q, s
 
 
 def num_threads():

@@ -702,6 +702,39 @@ EXPORT void orc_fp8_e8m0_gemv(const uint16_t* x, const uint8_t* w, const uint8_t
     free(W); free(xf);
 }
 
+/* FP8 E4M3 W [n, k] with one binary32 scale per output row; x binary32 [m, k], rounded to binary16 (act 0) or bf16 (act 1) or used
+ * as given (act 2); y[r, n] = (sum_k a(x) * w) * scale[n], rounded to binary16 when `rounded`.  The sum in binary64 (the products
+ * are exact; the reference's kernels sum in binary32, each in its own order), rounded once to binary32 before the scale, as the
+ * reference multiplies its finished binary32 sum.  reference engine-rs/shim/fp8.cu:13-22 (fp8_gemv), :110-151. */
+EXPORT void orc_fp8_rowscale_gemv(const float* x, const uint8_t* w, const float* scale, float* y, int m, int n, int k, int act, int rounded)
+{
+    float* xa = (float*)malloc((size_t)m * k * 4);
+    for (size_t i = 0; i < (size_t)m * k; ++i)
+        xa[i] = act == 0 ? orc_f16_to_f32(orc_f32_to_f16(x[i])) : act == 1 ? orc_bf16_to_f32(orc_f32_to_bf16(x[i])) : x[i];
+#pragma omp parallel for schedule(static)
+    for (int c = 0; c < n; ++c)
+        for (int r = 0; r < m; ++r) {
+            double acc = 0.0;
+            for (int j = 0; j < k; ++j) acc += (double)xa[(size_t)r * k + j] * (double)orc_e4m3_to_f32(w[(size_t)c * k + j]);
+            float v = (float)acc * scale[c];
+            if (rounded) v = orc_f16_to_f32(orc_f32_to_f16(v));
+            y[(size_t)r * n + c] = v;
+        }
+    free(xa);
+}
+/* The quantiser of that format: scale[n] = max(row amax, 1e-12) / 448, q = e4m3_rn(clamp(w / scale, +-448)), the division in
+ * binary32.  reference engine-rs/src/dense_fp8.rs:59-62 (quantize). */
+EXPORT void orc_fp8_rowscale_quant(const float* w, uint8_t* q, float* scale, int n, int k)
+{
+    for (int r = 0; r < n; ++r) {
+        float a = 0.f;
+        for (int j = 0; j < k; ++j) a = fmaxf(a, fabsf(w[(size_t)r * k + j]));
+        const float s = fmaxf(a, 1e-12f) / 448.0f;
+        scale[r] = s;
+        for (int j = 0; j < k; ++j) q[(size_t)r * k + j] = orc_f32_to_e4m3(fminf(fmaxf(w[(size_t)r * k + j] / s, -448.0f), 448.0f));
+    }
+}
+
 EXPORT int orc_num_threads(void)
 {
 #ifdef _OPENMP

@@ -99,6 +99,40 @@ int routes_check(const void* idx, bool idx64, int R, int topk, int E, hipStream_
 
 }  // namespace spk
 
+// ---- the stream floor: what this GPU needs to READ a number of bytes with nothing else to do.  Non-temporal 16-byte loads, eight in
+// flight a thread, over exactly `bytes` (rounded down to 16), one 4-byte store a wave: the time no kernel that must fetch those bytes
+// from memory can beat, measured the way the layer kernels are (the benchmark records it into the same graph of instances).  The
+// shape - 512 workgroups of 1024 threads walking the bytes with the grid's stride, all resident at once - is the fastest of the
+// shapes tried at 2 MB .. 326 MB (15.9 MB: 4.0 us against 6.1 for 256-thread workgroups that read eight pieces a thread and end).
+namespace spk {
+namespace {
+constexpr int SR_THREADS = 1024, SR_BLOCKS = 512;
+__global__ __launch_bounds__(SR_THREADS) void stream_read_kernel(const uint4* __restrict__ p, int64_t n16, uint32_t* __restrict__ out)
+{
+    const int64_t stride = (int64_t)gridDim.x * SR_THREADS;
+    int64_t i = (int64_t)blockIdx.x * SR_THREADS + threadIdx.x;
+    uint32_t acc = 0u;
+    for (; i + 7 * stride < n16; i += 8 * stride) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = ld_stream16(p + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    for (; i < n16; i += stride) { const uint4 v = ld_stream16(p + i); acc ^= v.x ^ v.y ^ v.z ^ v.w; }
+    acc ^= __float_as_uint(lane_xor<32>(__uint_as_float(acc), threadIdx.x & 63));
+    if ((threadIdx.x & 63) == 0) out[(blockIdx.x * (SR_THREADS / 64) + (threadIdx.x >> 6)) & 1023] = acc;
+}
+}  // namespace
+}  // namespace spk
+// src: device memory of `bytes` bytes (16-byte aligned), out: device memory of 4096 bytes
+SPARK_API int spark_debug_stream_read(const void* src, size_t bytes, void* out, hipStream_t st)
+{
+    if (!src || !out || bytes < 16 || ((uintptr_t)src & 15)) return 1;
+    spk::stream_read_kernel<<<spk::SR_BLOCKS, spk::SR_THREADS, 0, st>>>((const uint4*)src, (int64_t)(bytes / 16), (uint32_t*)out);
+    return spk::launch_status();
+}
+
 // diagnostics: 1 = check every call's routes on the host before launching (see routes_check), 0 = off, negative = as the environment says
 SPARK_API void spark_debug_validate_routes(int on) { spk::g_validate = on < 0 ? -1 : on ? 1 : 0; }
 

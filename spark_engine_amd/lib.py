@@ -82,10 +82,15 @@ SIGNATURES = {
     "glm_moe_experts": (i32, [vp, i64, i32, vp, vp, vp, vp, vp, vp, i32, vp, i32, vp]),
     "glm_moe3_ws_bytes": (sz, [i32, i32]),
     "glm_moe3_experts": (i32, [vp, i64, i32, vp, vp, vp, vp, vp, vp, i32, i32, vp]),
+    # weight-only FP8 with a scale per output row (the GLM dense projections)
+    "glm53_fp8_dense_cuda": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp]),
+    "glm53_fp8_bf16_cuda": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
+    "glm53_fp8_bf16_skinny_cuda": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
     # single-launch workspaces
     "spark_moe_ws_status": (i32, [vp, vp]),
     "spark_moe_ws_release": (None, [vp]),
     # diagnostics
+    "spark_debug_stream_read": (i32, [vp, sz, vp, vp]),
     "spark_debug_mx_ws_h": (i32, [vp, i32, i32, i32, i32, i32, i32, vp, vp, vp]),
     "spark_debug_exl3_local": (None, [i32]), "spark_debug_mx_local": (None, [i32]), "spark_debug_exl3_twa": (None, [i32]),
     "spark_debug_mx_out_cap": (None, [sz]), "spark_debug_validate_routes": (None, [i32]), "spark_mxfp4_moe_path": (i32, [i32] * 7), "spark_exl3_moe_path": (i32, [i32] * 6), "spark_debug_mx_fused_rows": (None, [i32]), "spark_debug_placement": (i32, []), "spark_debug_gemv_rows": (None, [i32]), "spark_debug_fp8q_rowmajor": (None, [i32]),

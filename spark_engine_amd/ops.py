@@ -357,6 +357,32 @@ def fp8_e8m0_gemv_t16(x, wt, scales, n, y=None):
     return y
 
 
+def fp8_rowscale_quantize(w):
+    """reference engine-rs/src/dense_fp8.rs:59-62 (quantize): one scale per output row = row amax / 448, codes = E4M3 of w / scale.
+    w [n, k] f32 | f16 | bf16 -> (E4M3 bytes [n, k] as uint8, scales f32 [n])."""
+    wf = w.float()
+    # the two binary32 divisions through binary64 (correctly rounded either way: a device division may be a multiplication by 1 / 448)
+    scale = (wf.abs().amax(dim=1, keepdim=True).clamp_min(1e-12).double() / 448.0).float()
+    q = (wf.double() / scale.double()).float().clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    return q.view(torch.uint8), scale.view(-1).contiguous()
+
+
+def glm_fp8_dense(x, wq, scales, rounded=False, act="f16"):
+    """reference engine-rs/src/dense_fp8.rs run / cached -> glm53_fp8_dense_cuda (act f16) | glm53_fp8_bf16_cuda (act bf16) |
+    glm53_fp8_bf16_skinny_cuda (x given as bf16): x [m, k] -> y f32 [m, n]."""
+    m, k = x.shape
+    n = wq.shape[0]
+    y = torch.empty(m, n, dtype=torch.float32, device=x.device)
+    L = _lib()
+    if x.dtype == torch.bfloat16:
+        _ck(L.glm53_fp8_bf16_skinny_cuda(_p(_dev(x)), _p(_dev(wq)), _p(_dev(scales)), _p(y), m, n, k, _st()), "glm53_fp8_bf16_skinny_cuda")
+    elif act == "bf16":
+        _ck(L.glm53_fp8_bf16_cuda(_p(_dev(x)), _p(_dev(wq)), _p(_dev(scales)), _p(y), None, m, n, k, 1, _st()), "glm53_fp8_bf16_cuda")
+    else:
+        _ck(L.glm53_fp8_dense_cuda(_p(_dev(x)), _p(_dev(wq)), _p(_dev(scales)), _p(y), None, m, n, k, int(rounded), 1, 0, _st()), "glm53_fp8_dense_cuda")
+    return y
+
+
 def bf16_gemv(x, w):
     m, k = x.shape
     n = w.shape[0]

@@ -169,6 +169,38 @@ def test_requant_fp8_vs_library(oracle):
     assert s1[0, 0] == 122 and q1[0, 0] == 0x78 and q1[0, 1] == 0xfc and not q1[0, 2:].any()
 
 
+# ---------------------------------------------------------------- weight-only FP8 with a scale per output row (GLM dense projections)
+
+def test_fp8_rowscale_quant_and_gemv_vs_library(oracle):
+    # quantiser (reference dense_fp8.rs:59-62) against torch's own float8 cast, the product against a binary64 matmul of the library's
+    # f16 / bf16 roundings; hand-worked values pin the scale rule and the order "sum, then scale, then round"
+    g = torch.Generator().manual_seed(11)
+    n, k, m = 96, 320, 5
+    w = torch.randn(n, k, generator=g) * (10.0 ** torch.empty(n, 1).uniform_(-3, 2, generator=g))
+    w[7] = 0.0                                                          # an all-zero row: the scale floor 1e-12 / 448, codes 0
+    q, s = oracle.fp8_rowscale_quant(w.numpy())
+    s_ref = (w.abs().amax(dim=1).clamp_min(1e-12) / 448.0)
+    assert np.array_equal(s, s_ref.numpy())
+    q_ref = (w / s_ref[:, None]).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(q, q_ref)
+    assert (np.abs(torch.from_numpy(q).view(torch.float8_e4m3fn).float().numpy()).max(axis=1)[np.arange(n) != 7] == 448.0).all()   # every row uses the full range
+    x = torch.randn(m, k, generator=g) * 3.0
+    wd = torch.from_numpy(q).view(torch.float8_e4m3fn).double()
+    for act, cast in ((0, torch.float16), (1, torch.bfloat16)):
+        ref = ((x.to(cast).double() @ wd.T).float() * torch.from_numpy(s)[None]).numpy()
+        got = oracle.fp8_rowscale_gemv(x.numpy(), q, s, act=act)
+        assert np.array_equal(got, ref)                                 # binary64 sums of exact products: the same value whatever the order
+        assert not np.array_equal(got, oracle.fp8_rowscale_gemv(x.numpy(), q, s, act=2))          # the rounding of the activations is there
+    rounded = oracle.fp8_rowscale_gemv(x.numpy(), q, s, act=0, rounded=True)
+    ref = ((x.half().double() @ wd.T).float() * torch.from_numpy(s)[None]).half().float().numpy()
+    assert np.array_equal(rounded, ref)
+    # by hand: w row (2, -1), x (3, 5) -> scale 2 / 448, codes 448 and -224, sum 3 * 448 - 5 * 224 = 224, y = 224 * 2 / 448 = 1
+    q1, s1 = oracle.fp8_rowscale_quant(np.array([[2.0, -1.0] + [0.0] * 6], np.float32))
+    assert s1[0] == np.float32(2.0) / np.float32(448.0) and q1[0, 0] == 0x7e and q1[0, 1] == 0xf6
+    y1 = oracle.fp8_rowscale_gemv(np.array([[3.0, 5.0] + [0.0] * 6], np.float32), q1, s1, act=0)
+    assert abs(y1[0, 0] - 1.0) < 1e-6
+
+
 # ---------------------------------------------------------------- shared-expert glue
 
 def test_swiglu_quant_vs_float64_and_act_quant(oracle):
