@@ -250,6 +250,10 @@ SPARK_API int spark_exl3_moe(const void* x, int xtype, int64_t ldx, int R, const
  * call's leftovers.  All calls on one GPU share the array: calls that overlap on one GPU race. */
 SPARK_API int spark_exl3_moe_static(const void* x, int xtype, int64_t ldx, int R, const void* idx, int itype, const void* w, int wtype, const void* tab,
                                     const void* add, void* out, int H, int I, int E, int topk, int codebook, int act, hipStream_t st);
+/* The error flag of that array after the last spark_exl3_moe_static call on the current device (each call clears it as it starts):
+ * waits for the stream, then 0 = every wait of the call was served, 1 = a wait expired or the routes broke the contract (the rows
+ * concerned hold NaN), negative = not set up / the read failed.  Synchronises: a diagnostic, never on a capturing stream. */
+SPARK_API int spark_exl3_moe_static_status(hipStream_t st);
 /* Qwen: E 512, top-10, H 2560, I 640, x / w fp32, idx int32, mul1.  Replaces engine-rs/shim/qwen_moe.cu:111-117.
  * S (here and in the glm_* forms) is the reference's K-slice count, a tuning hint there: accepted and ignored, the slices follow the
  * shape alone so that a row's bits do not depend on the call. */
@@ -274,11 +278,15 @@ SPARK_API int glm_moe3_experts(const void* x, int64_t ldx, int R, const void* id
 
 /* The single-launch decode kernels (spark_exl3_moe, spark_mxfp4_moe_x and the reference-named forms at up to 8 rows) pass data
  * between the workgroups of one launch through words of ws that are all-ones while idle; every wait is bounded.  If a wait ever
- * expires (it never should: a block only waits for blocks dispatched before it), the kernel sets the first 32-bit word of ws, stores
- * nothing for the rows concerned and still runs to its end; the launch returns 0 like the reference's launchers, which cannot see
- * device state either.  spark_moe_ws_status(ws, st) waits for st and returns that flag: 0 = no wait has expired since ws was
- * prepared, 1 = one has (prepare ws again with the matching *_ws_init before the next call), negative = the read failed.  It
- * synchronises: a diagnostic for tests, benchmarks and a serving loop's periodic health check, not for captured streams.
+ * expires (it never should: a block only waits for blocks dispatched before it), or a token row names an expert twice (an item
+ * would outgrow the kernels' arrays: it is cut at what they hold), the kernel sets the first 32-bit word of ws (sticky), stores NaN
+ * into every output element whose sum it could not complete and still runs to its end; the launch returns 0 like the reference's
+ * launchers, which cannot see device state either, so the failure is in the data for a caller that only checks return codes.  While
+ * the flag is set every later call on that workspace stores NaN too (the words a failed call left behind are not idle), until the
+ * workspace is prepared again.  spark_moe_ws_status(ws, st) waits for st and returns the flag: 0 = clear, 1 = set - and ws is then
+ * no longer known as prepared, so the next call that does not pass "prepared" (flags bit 0) prepares it again itself; a caller that
+ * passes the bit calls the matching *_ws_init first -, negative = the read failed.  It synchronises: a diagnostic for tests,
+ * benchmarks and a serving loop's periodic health check, not for captured streams.
  * spark_moe_ws_release(ws): forget that ws was prepared (before freeing or reusing the memory). */
 SPARK_API int spark_moe_ws_status(const void* ws, hipStream_t st);
 SPARK_API void spark_moe_ws_release(const void* ws);

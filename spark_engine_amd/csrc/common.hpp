@@ -220,9 +220,12 @@ template <int NJ, class F> __device__ __forceinline__ void wave_items_init(WaveI
         base += __builtin_popcountll(m);
     }
 }
-// item g: its expert (or -1 when the call has fewer items), its pairs in rows[0 .. n)
-template <int NJ> __device__ __forceinline__ int wave_items_pick(const WaveItems<NJ>& w, int g, int lane, int* rows, int& n)
+// item g: its expert (or -1 when the call has fewer items), its pairs in rows[0 .. n).  cap: the entries rows[] has; an item with more
+// pairs than that (only possible when a token row names an expert twice, which the routes' contract excludes) keeps its first cap
+// pairs, n stops at cap and `over` is set: the caller raises the workspace's error flag instead of writing past its arrays.
+template <int NJ> __device__ __forceinline__ int wave_items_pick(const WaveItems<NJ>& w, int g, int lane, int* rows, int& n, int cap, bool& over)
 {
+    over = false;
     int eg = -1;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
@@ -235,9 +238,10 @@ template <int NJ> __device__ __forceinline__ int wave_items_pick(const WaveItems
     for (int j = 0; j < NJ; ++j) {
         const bool hit = w.e[j] == eg;
         const uint64_t m = __builtin_amdgcn_ballot_w64(hit);
-        if (hit) rows[n + lanes_below(m)] = lane + 64 * j;
+        if (hit && n + lanes_below(m) < cap) rows[n + lanes_below(m)] = lane + 64 * j;
         n += __builtin_popcountll(m);
     }
+    if (n > cap) { n = cap; over = true; }
     return eg;
 }
 
@@ -257,9 +261,11 @@ __device__ __forceinline__ void st_stream16(void* p, uint4 v)
 }
 
 // A routing index as the kernels use it: forced into [0, E - 1], so that an index far outside the table cannot become an address far
-// outside the weights.  Valid routes are unchanged.  This does not make invalid routes safe: the kernels' contract is the
-// reference's - every index in range and the experts of one token row distinct (an item then never holds more rows than the call) -
-// and routes read before the router has written them (a caller's stream race) break it whatever the clamp does.
+// outside the weights.  Valid routes are unchanged.  The kernels' contract is the reference's - every index in range and the experts
+// of one token row distinct (an item then never holds more rows than the call).  Routes that break it (NaN logits in a caller's router,
+// indices read before the router has written them) stay inside the kernels' arrays all the same: the clamp bounds the index, the
+// single-launch kernels cap an item's rows at what their arrays hold (wave_items_pick) and raise the workspace's error flag, and the
+// rows concerned come out as NaN.
 __device__ __forceinline__ int clamp_expert(int e, int E) { return min(max(e, 0), E - 1); }
 
 inline int launch_status() { return (int)hipGetLastError(); }

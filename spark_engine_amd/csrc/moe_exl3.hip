@@ -349,12 +349,18 @@ __global__ __launch_bounds__(64 * GV_WAVES) void item_kernel(const uint16_t* __r
     __shared__ uint32_t tw[MIXED ? 8 * 48 : 8];
     const int g = blockIdx.y, nb = blockIdx.x;
     if (g >= *G) return;
-    const int rows = gcnt[g], e = gexp[g], row0 = goff[g];
+    // the host asks the grouping for items of at most this instance's rows (gr_of_rows), so the bound never bites; it stays as the
+    // guarantee that the arrays below cannot be overrun whatever the grouping wrote
+    const int rows = min(gcnt[g], SR), e = gexp[g], row0 = goff[g];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int bits = MIXED ? (int)tab[(int64_t)9 * E + e] : 4;
+    const int bits_raw = MIXED ? (int)tab[(int64_t)9 * E + e] : 4;
+    // a width the format does not have (row 9 outside 3..6): the expert contributes nothing - its products run over no k-tiles, so its
+    // rows are finished and stored as zeros like any others (nothing downstream reads memory nobody wrote)
+    const bool bits_ok = bits_raw >= 3 && bits_raw <= 6;
+    const int bits = bits_ok ? bits_raw : 4;
     // vw: the expert's own intermediate width replaces N (gate / up) or K (down); strides keep N / K
     const int we = vw ? (int)tab[(int64_t)10 * E + e] : 0;
-    const int Ne = vw && STAGE == 1 ? we : N, Ke = vw && STAGE == 2 ? we : K;
+    const int Ne = vw && STAGE == 1 ? we : N, Ke = !bits_ok ? 0 : vw && STAGE == 2 ? we : K;
     if (nb * 128 >= Ne) return;
     const int n = nb * 128 + 2 * lane;
     if constexpr (STAGE == 1) {
@@ -540,7 +546,7 @@ __global__ __launch_bounds__(256, 6) void gemm_kernel(const uint16_t* __restrict
                 case 4: gemm_pass<CBK, KT, 4>(xrows, K, rows, Ke, tr, Ne / 16, nb, smem, acc); break;
                 case 5: gemm_pass<CBK, KT, 5>(xrows, K, rows, Ke, tr, Ne / 16, nb, smem, acc); break;
                 case 6: gemm_pass<CBK, KT, 6>(xrows, K, rows, Ke, tr, Ne / 16, nb, smem, acc); break;
-                default: return;                                // a width the format does not have: nothing stored
+                default: break;                                 // a width the format does not have: the expert contributes nothing, zeros are stored
             }
         }
     }
@@ -639,7 +645,11 @@ inline Plan plan(const Cfg& c, int R, int GR)
     p.total = o;
     return p;
 }
-constexpr int GR_ITEM = 16;            // rows of an item of the item kernels
+constexpr int GR_ITEM = 16;            // most rows of an item of the item kernels
+// Rows of an item for a call of R rows = the row count of the kernel instance the call runs (1, 2, 4, 8, 16).  With valid routes an
+// expert has at most R rows anyway; a token row that names an expert twice then gives that expert a second item instead of an item
+// larger than the instance's arrays, and its pairs are all multiplied and summed.
+inline int gr_of_rows(int R, bool mixed) { return mixed || R > 8 ? GR_ITEM : R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : 8; }
 inline bool cfg_ok(const Cfg& c, int R)
 {
     return R >= 1 && c.E >= 1 && c.E <= EMAX && c.topk >= 1 && c.topk <= 64 && (int64_t)R * c.topk <= PMAX && R <= 64 && c.H >= 128 && c.I >= 128 &&
@@ -683,7 +693,8 @@ int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, co
         cf.varw = varw ? 1 : 0;
         return exl3_fused_launch(cf, x, ldx, R, idx, w, tab, add, out, ws, flags & 1, st);
     }
-    const Plan p = plan(c, R, GR_ITEM);
+    const int gr = gr_of_rows(R, mixed);
+    const Plan p = plan(c, R, gr);
     char* b = (char*)ws + fused_cap(c);              // the two paths never share workspace bytes
     int* G = (int*)(b + p.G);
     int *gexp = (int*)(b + p.gexp), *goff = (int*)(b + p.goff), *gcnt = (int*)(b + p.gcnt);
@@ -693,7 +704,7 @@ int experts(const Cfg& c, const void* x, int64_t ldx, int R, const void* idx, co
     float* pout = (float*)(b + p.pout);
     const uint64_t* tb = (const uint64_t*)tab;
     const int maxrows = R < GR_ITEM ? R : GR_ITEM, vw = varw ? 1 : 0;
-    group_pairs_kernel<<<1, 1024, 0, st>>>(idx, c.itype, R, c.topk, c.E, GR_ITEM, G, gexp, goff, gcnt, pairmap, ppair, pexp, nullptr, nullptr);
+    group_pairs_kernel<<<1, 1024, 0, st>>>(idx, c.itype, R, c.topk, c.E, gr, G, gexp, goff, gcnt, pairmap, ppair, pexp, nullptr, nullptr);
     const int64_t waves = (int64_t)2 * p.P;
     // x rows on 16-byte boundaries (every layout the callers have): whole 16-byte reads
     if ((uintptr_t)x % 16 == 0 && ldx % (c.xtype == X_F32 ? 4 : 8) == 0)
@@ -823,6 +834,7 @@ SPARK_API size_t spark_exl3_moe_ws_bytes(int R, int H, int I, int E, int topk)
     const int n = R < RC ? R : RC;                   // rows of the largest pass
     if (!cfg_ok(c, n)) return 0;
     size_t need = plan(c, n, GR_ITEM).total;
+    { const size_t v = plan(c, n, gr_of_rows(n, false)).total; if (v > need) need = v; }     // uniform tables group by the instance's row count
     if (big_ok(c, R)) { const size_t v = plan(c, R, PG_ROWS).total; if (v > need) need = v; }
     return fused_cap(c) + need;                      // grows with R: a caller may size once for its largest call
 }

@@ -138,7 +138,8 @@ __device__ __forceinline__ int ld_idx_k(const void* idx, int itype, int i) { ret
 struct Group { int e, n; };
 // item g of the call: expert and its pair rows (ascending) in rows[], or n = 0 when the call has fewer items.  All threads
 // call; wave 0 works the item out (one barrier).
-__device__ __forceinline__ Group find_item(const FArgs& a, int g, int* owner, int* rows, int* misc)
+// cap: the rows this kernel instance's arrays hold per item (MR); an item beyond it is cut there and the error flag raised.
+__device__ __forceinline__ Group find_item(const FArgs& a, int g, int* owner, int* rows, int* misc, int cap)
 {
     const int P = a.P, tid = threadIdx.x;
     if (a.R == 1) {                                       // every pair is its own item
@@ -152,8 +153,9 @@ __device__ __forceinline__ Group find_item(const FArgs& a, int g, int* owner, in
         WaveItems<PF_MAX / 64> wi;
         wave_items_init(wi, P, tid, owner, [&](int p) { return clamp_expert(exl3_ld_idx(a.idx, a.c.itype, p), a.c.E); });
         int n = 0;
-        const int e = wave_items_pick(wi, g, tid, rows, n);
-        if (tid == 0) { misc[0] = e; misc[1] = n; }
+        bool over;
+        const int e = wave_items_pick(wi, g, tid, rows, n, cap, over);
+        if (tid == 0) { misc[0] = e; misc[1] = n; if (over) atomicExch(a.err, 1); }
     }
     __syncthreads();
     return misc[0] < 0 ? Group{0, 0} : Group{__builtin_amdgcn_readfirstlane(misc[0]), __builtin_amdgcn_readfirstlane(misc[1])};
@@ -203,7 +205,12 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
     }
     if (tid == 0) misc[2] = 1;
     Group grp{0, 0};
-    if (g >= 0) grp = find_item(a, g, owner, rows, misc);
+    if (g >= 0) grp = find_item(a, g, owner, rows, misc, MR);
+    // The summing blocks look at the workspace's error flag as they start: it is sticky, so a wait that expired in an EARLIER call (which
+    // left words of the workspace behind that are not idle) turns every later call's output into NaN until the workspace is prepared
+    // again, instead of sums of stale words.  The load is in flight while the block waits for its slices.
+    int stale = 0;
+    if (isC && s) stale = __hip_atomic_load(a.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // Experts with their own intermediate width (row 10 of the table, reference moe_exl3.cuh:63-67,132-136): fewer column blocks in
     // gate / up (the blocks past the width have no work and their group exchanges nothing), fewer k-tiles in down; the exchange
     // buffers keep the strides of the widest expert.
@@ -240,10 +247,17 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
             red[wave][0][2 * lane] = a0; red[wave][0][2 * lane + 1] = a1;
             __syncthreads();
             if (!ok && lane == 0) atomicExch(a.err, 1);
-            if (wave == 0 && ok) {
+            misc[3] = 1;
+            __syncthreads();
+            if (!ok || stale) misc[3] = 0;                // any wave's wait expired, or the workspace was not idle when the call began
+            __syncthreads();
+            if (wave == 0) {
                 float v0 = red[0][0][2 * lane], v1 = red[0][0][2 * lane + 1];
 #pragma unroll
                 for (int w = 1; w < FW; ++w) { v0 += red[w][0][2 * lane]; v1 += red[w][0][2 * lane + 1]; }
+                // a failed call must not leave the caller's old bytes in out, where a caller that only looks at the return code would
+                // take them for a result: every column this block owns becomes NaN (every upstream failure ends here as an expired wait)
+                if (!misc[3]) { v0 = __uint_as_float(0x7fc00000u); v1 = v0; }
                 if (c.obf16) *(uint32_t*)((uint16_t*)a.out + (int64_t)t * c.H + ncol) = (uint32_t)f32_to_bf16(b0 + v0) | ((uint32_t)f32_to_bf16(b1 + v1) << 16);
                 else { a.out[(int64_t)t * c.H + ncol] = b0 + v0; a.out[(int64_t)t * c.H + ncol + 1] = b1 + v1; }
             }

@@ -3,6 +3,7 @@
 #include "moe_exl3.hpp"
 #include "runtime.hpp"
 #include "exl3_decode.hpp"
+#include <atomic>
 
 namespace spk {
 
@@ -10,7 +11,8 @@ namespace {
 constexpr size_t SCRATCH_BYTES = (size_t)16 << 20;        // the largest single-launch call it takes (the 512-expert top-10 layer at 8 rows needs 5.3 MB)
 static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
 constexpr int MAX_DEVICES = 64;
-void* g_scratch_ptr[MAX_DEVICES] = {};                    // per device: every GPU holds its own copy of the array at its own address
+std::atomic<void*> g_scratch_ptr[MAX_DEVICES] = {};       // per device: every GPU holds its own copy of the array at its own address (two
+                                                          // host threads that set up the same device store the same address)
 }  // namespace
 
 // the array's device address on the current device, resolved once per device (the name `scratch` itself is a host-side stand-in)
@@ -20,12 +22,12 @@ int exl3_static_setup()
     hipError_t rc = hipGetDevice(&dev);
     if (rc != hipSuccess) return (int)rc;
     if (dev < 0 || dev >= MAX_DEVICES) return -6;
-    if (g_scratch_ptr[dev]) return 0;
+    if (g_scratch_ptr[dev].load()) return 0;
     void* ptr = nullptr;
     rc = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (rc != hipSuccess) return (int)rc;
     if (!ptr) return -6;
-    g_scratch_ptr[dev] = ptr;
+    g_scratch_ptr[dev].store(ptr);
     return 0;
 }
 
@@ -47,7 +49,20 @@ extern "C" __attribute__((visibility("default"))) int spark_exl3_moe_static(cons
     if (rs) return rs;
     int dev = 0;
     (void)hipGetDevice(&dev);
-    return exl3_fused_launch(c, x, ldx, R, idx, w, tab, add, out, g_scratch_ptr[dev], 0, st);
+    return exl3_fused_launch(c, x, ldx, R, idx, w, tab, add, out, g_scratch_ptr[dev].load(), 0, st);
+}
+
+// The error flag of the library's own array after the last spark_exl3_moe_static call on the current device (every call clears it as
+// it starts): waits for the stream, then 0 = every wait of that call was served, 1 = a wait expired or the routes broke the contract
+// (the rows concerned hold NaN), negative = the array is not set up or the read failed.  Synchronises: never on a capturing stream.
+extern "C" __attribute__((visibility("default"))) int spark_exl3_moe_static_status(hipStream_t st)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES || !g_scratch_ptr[dev].load()) return -1;
+    if (hipStreamSynchronize(st) != hipSuccess) return -2;
+    int flag = 0;
+    if (hipMemcpy(&flag, g_scratch_ptr[dev].load(), sizeof(flag), hipMemcpyDeviceToHost) != hipSuccess) return -3;
+    return flag != 0 ? 1 : 0;
 }
 
 }  // namespace spk

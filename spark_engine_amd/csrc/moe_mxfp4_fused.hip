@@ -125,9 +125,10 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
 #pragma unroll
             for (int j = 0; j < PMAXF / 64; ++j) if (lane + 64 * j < a.P) sidx[lane + 64 * j] = wi.e[j];
             int nu = 0, nd = 0;
-            const int eu = wantU ? wave_items_pick(wi, grpi, lane, rowsU, nu) : -1;
-            const int ed = wantD ? wave_items_pick(wi, grpi - 1, lane, rowsD, nd) : -1;
-            if (lane == 0) { gsel[0] = eu; gsel[1] = nu; gsel[2] = ed; gsel[3] = nd; }
+            bool ou = false, od = false;                   // an item never holds more rows than the call unless a token row names an expert twice
+            const int eu = wantU ? wave_items_pick(wi, grpi, lane, rowsU, nu, a.R, ou) : -1;
+            const int ed = wantD ? wave_items_pick(wi, grpi - 1, lane, rowsD, nd, a.R, od) : -1;
+            if (lane == 0) { gsel[0] = eu; gsel[1] = nu; gsel[2] = ed; gsel[3] = nd; if (ou || od) atomicExch(a.err, 1); }
         }
         __syncthreads();
         gu = Group{gsel[0], gsel[0] >= 0 ? gsel[1] : 0};
@@ -401,6 +402,17 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
     // the other blocks' weight rows)
     float base = 0.f;
     if (wave < grp.n && comb[wave] && a.add) base = a.add[(int64_t)(rows[wave] / a.TT) * H + nb * DC + lane];
+    // The summing waves look at the workspace's error flag as they start: it is sticky, so a wait that expired in an EARLIER call (which
+    // left words behind that are not idle) turns every later call's output into NaN until the workspace is prepared again.
+    int stale = 0;
+    if (wave < grp.n && comb[wave]) stale = __hip_atomic_load(a.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // a failed call must not leave the caller's old bytes in y: the columns this wave owns become NaN
+    auto poison = [&]() {
+        if (wave < grp.n && comb[wave]) {
+            const int64_t o = (int64_t)(rows[wave] / a.TT) * H + nb * DC + lane;
+            if (a.obf16) ((uint16_t*)a.y)[o] = 0x7fc0u; else a.y[o] = __uint_as_float(0x7fc00000u);
+        }
+    };
     // B operands of a round in LDS: [kw][step][g4][row < n] x (8 code words + 1 scale word), written by the waves of half 0
     uint32_t* hl = (uint32_t*)extra;
     const bool valid = c < grp.n;
@@ -486,7 +498,7 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
         }
     }
     TRACE(8);
-    if (!misc[2]) { if (tid == 0) atomicExch(a.err, 1); return; }
+    if (!misc[2]) { if (tid == 0) atomicExch(a.err, 1); poison(); return; }
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -527,7 +539,7 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
             if (++spins >= SPIN_MAX) { ok = false; break; }
             __builtin_amdgcn_s_sleep(1);
         }
-        if (ok) {
+        if (ok && !stale) {
 #pragma unroll
             for (int k = 0; k < TTMAX; ++k) { if (LOCAL) *(uint32_t*)py[k] = EMPTY; else st_dev32(py[k], EMPTY); }
             float accs = base;                             // add + shared experts, then the routed experts in slot order
@@ -538,7 +550,7 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
             for (int k = 0; k < TTMAX; ++k) if (k < a.topk) s += __uint_as_float(o[k]);
             if (a.obf16) ((uint16_t*)a.y)[(int64_t)tok * H + col] = f32_to_bf16(accs + s);
             else a.y[(int64_t)tok * H + col] = accs + s;
-        } else if (lane == 0) atomicExch(a.err, 1);
+        } else { poison(); if (lane == 0) atomicExch(a.err, 1); }
     }
     TRACE(10);
 }

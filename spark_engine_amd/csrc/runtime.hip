@@ -2,6 +2,7 @@
 // their owner has prepared, and the read-out of a workspace's bounded-wait flag.
 #include "runtime.hpp"
 
+#include <atomic>
 #include <cstdlib>
 #include <mutex>
 #include <unordered_map>
@@ -20,8 +21,9 @@ __global__ void xcd_probe_kernel(int* out)
     if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((31 << 11) | 20) & 0xf;
 }
 
-int g_placement = -1;                  // -1 not checked yet, 0 check failed, 1 workgroup b of a 1-D grid runs on XCD b % 8
-std::mutex g_mu;
+std::atomic<int> g_placement{-1};      // -1 not checked yet, 0 check failed, 1 workgroup b of a 1-D grid runs on XCD b % 8.  One value for the
+                                       // process: the property belongs to the GPU model and the runtime, and every GPU of a node is the same model
+std::mutex g_mu, g_probe_mu;
 std::unordered_map<const void*, size_t> g_prepared;       // workspace base -> bytes its owner prepared
 
 }  // namespace
@@ -31,6 +33,8 @@ std::unordered_map<const void*, size_t> g_prepared;       // workspace base -> b
 // device-coherent accesses only.
 int xcd_placement_check()
 {
+    if (g_placement >= 0) return g_placement;
+    std::lock_guard<std::mutex> lk(g_probe_mu);            // two host threads: one runs the check, the other finds its result
     if (g_placement >= 0) return g_placement;
     int* d = nullptr;
     if (hipGetSymbolAddress((void**)&d, HIP_SYMBOL(g_probe)) != hipSuccess) return g_placement = 0;
@@ -145,6 +149,7 @@ SPARK_API int spark_moe_ws_status(const void* ws, hipStream_t st)
     if (hipStreamSynchronize(st) != hipSuccess) return -2;
     int flag = 0;
     if (hipMemcpy(&flag, ws, sizeof(flag), hipMemcpyDeviceToHost) != hipSuccess) return -3;
+    if (flag != 0) spk::ws_forget(ws);                     // no longer known as prepared: the next call that may prepare it does so itself
     return flag != 0 ? 1 : 0;
 }
 // The owner of a prepared workspace is about to free it (or hand it to other code): calls through the reference-named entry points

@@ -87,7 +87,7 @@ SIGNATURES = {
     "glm53_fp8_bf16_cuda": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
     "glm53_fp8_bf16_skinny_cuda": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
     # single-launch workspaces
-    "spark_moe_ws_status": (i32, [vp, vp]),
+    "spark_moe_ws_status": (i32, [vp, vp]), "spark_exl3_moe_static_status": (i32, [vp]),
     "spark_moe_ws_release": (None, [vp]),
     # diagnostics
     "spark_debug_stream_read": (i32, [vp, sz, vp, vp]),

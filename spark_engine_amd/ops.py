@@ -496,23 +496,25 @@ def moe_pack_mx(wp):
 
 
 def moe_scales_s2(sp):
-    """reference kern.rs moe_scales_s2: tile-packed scales [E, rows, K/32] (moe_pack) -> the lossless 2-bit coded blob
-    (desc [tiles][16] | codes [tiles][steps][8] | raw words of the tiles with a row spanning more than 3), uint8.
-    Returns (blob, raw tiles, tiles)."""
-    e, rows, nb = sp.shape
-    tiles, steps = e * rows // 8, nb // 4
-    v = sp.view(tiles, steps, 8, 4).to(torch.int16)
-    mn = v.amin(dim=(1, 3))                                             # [tiles, 8]
-    raw = ((v.amax(dim=(1, 3)) - mn) > 3).any(dim=1)                    # [tiles]
-    code = (v - mn.view(tiles, 1, 8, 1)).clamp(0, 3)
-    wts = torch.tensor([1, 4, 16, 64], dtype=torch.int16, device=sp.device).view(1, 1, 1, 4)
-    cb = (code * wts).sum(dim=3).to(torch.uint8).contiguous()           # [tiles, steps, 8]
-    ri = raw.to(torch.int32).cumsum(0).to(torch.int32) - 1
-    ri = torch.where(raw, ri, torch.full_like(ri, -1)).contiguous()
-    rawt = sp.view(tiles, steps * 32)[raw]
-    desc = torch.cat([mn.to(torch.uint8), ri.view(torch.uint8).view(tiles, 4), torch.zeros(tiles, 4, dtype=torch.uint8, device=sp.device)], dim=1)
-    blob = torch.cat([desc.reshape(-1), cb.reshape(-1), rawt.contiguous().reshape(-1)])
-    return blob.contiguous(), int(raw.sum().item()), tiles
+    """The 2-bit scale blob the ds41_moe_mx* entry points read after moe_s2_set(True) (the format of reference
+    engine-rs/shim/ds41_mx.cu:64-91, written there by kern.rs moe_scales_s2).  sp: tile-packed scale bytes [E, rows, K/32] from
+    moe_pack.  Per 8-row tile the blob holds a 16-byte descriptor (the eight rows' smallest scale byte, then a little-endian int32:
+    the tile's position among the raw tiles, or -1), per tile and 128-wide K step eight code bytes (one per row: the four blocks'
+    offsets above the row's smallest byte, two bits each, block 0 lowest), and, for tiles with a row whose bytes span more than 3, the
+    tile's raw bytes.  Lossless.  Returns (blob uint8, number of raw tiles, number of tiles)."""
+    n_exp, rows, n_blocks = sp.shape
+    n_tiles, n_steps = n_exp * rows // 8, n_blocks // 4
+    t = sp.reshape(n_tiles, n_steps, 8, 4)                               # [tile][K step][row of the tile][32-block of the step]
+    row_min = t.amin(dim=(1, 3))                                         # [tile][row]
+    keeps_raw = (t.amax(dim=(1, 3)).int() - row_min.int() > 3).any(dim=1)
+    offs = (t - row_min[:, None, :, None]).clamp(max=3)                  # uint8; meaningless (and unread) in raw tiles
+    code_bytes = offs[..., 0] | (offs[..., 1] << 2) | (offs[..., 2] << 4) | (offs[..., 3] << 6)
+    raw_pos = torch.where(keeps_raw, torch.cumsum(keeps_raw.int(), 0) - 1, torch.full((n_tiles,), -1, device=sp.device)).to(torch.int32)
+    desc = torch.zeros(n_tiles, 16, dtype=torch.uint8, device=sp.device)
+    desc[:, :8] = row_min
+    desc[:, 8:12] = raw_pos.contiguous().view(torch.uint8).view(n_tiles, 4)
+    blob = torch.cat([desc.reshape(-1), code_bytes.contiguous().reshape(-1), t[keeps_raw].reshape(-1)])
+    return blob.contiguous(), int(keeps_raw.sum().item()), n_tiles
 
 
 def moe_s2_set(on):
@@ -560,6 +562,14 @@ class ExpertTable:
         variable-width tables (moe_exl3.cuh:63-67,132-136)."""
         self.E = E
         self.keep = experts
+        if bits is not None:
+            wrong = {e: b for e, b in bits.items() if int(b) not in (3, 4, 5, 6)}
+            if wrong:
+                raise ValueError(f"trellis widths are 3..6 bits: {wrong}")
+        if widths is not None:
+            wrong = {e: v for e, v in widths.items() if int(v) < 128 or int(v) % 128}
+            if wrong:
+                raise ValueError(f"an expert's intermediate width is a positive multiple of 128: {wrong}")
         rows = [[0] * E for _ in range(11 if widths is not None else 9 if bits is None else 10)]
         for e, ts in experts.items():
             for slot, t in enumerate(ts):

@@ -87,3 +87,71 @@ def test_fixed_width_entry_points_reject_other_widths():
         ops.ds41_moe_mx(xq, xs, idx, rw, w, 128)
     with pytest.raises(ValueError):
         ops.ds41_moe(torch.zeros(2, 1024, dtype=torch.bfloat16), idx, rw, w, 128)
+
+
+def _wave_items(experts, cap, nj=2):
+    """Restatement of the one-wave item logic of the single-launch kernels (wave_items_init / wave_items_pick: lane l holds pairs
+    l, l + 64, ...; an owner table gives every expert its first pair; ballots rank the first pairs and collect an item's pairs) as
+    the 64 lanes execute it, with the cap on an item's rows.  -> list of (expert, rows written, n reported, over)."""
+    P = len(experts)
+    e = [[experts[l + 64 * j] if l + 64 * j < P else -1 for j in range(nj)] for l in range(64)]
+    owner = {}
+    for l in range(64):
+        for j in range(nj):
+            if e[l][j] >= 0:
+                owner[e[l][j]] = min(owner.get(e[l][j], 1 << 30), l + 64 * j)
+    first = [[e[l][j] >= 0 and owner[e[l][j]] == l + 64 * j for j in range(nj)] for l in range(64)]
+    rank, base = [[0] * nj for _ in range(64)], 0
+    for j in range(nj):
+        m = [first[l][j] for l in range(64)]
+        for l in range(64):
+            rank[l][j] = base + sum(m[:l])
+        base += sum(m)
+    out = []
+    for g in range(base + 1):
+        eg = -1
+        for j in range(nj):
+            hit = [l for l in range(64) if first[l][j] and rank[l][j] == g]
+            if hit:
+                eg = e[hit[0]][j]
+        if eg < 0:
+            out.append((-1, [], 0, False))
+            continue
+        rows, n = [None] * cap, 0
+        for j in range(nj):
+            m = [e[l][j] == eg for l in range(64)]
+            for l in range(64):
+                if m[l] and n + sum(m[:l]) < cap:
+                    assert 0 <= n + sum(m[:l]) < cap                        # the store the kernel makes: always inside rows[cap]
+                    rows[n + sum(m[:l])] = l + 64 * j
+            n += sum(m)
+        over = n > cap
+        out.append((eg, rows[:min(n, cap)], min(n, cap), over))
+    return out
+
+
+def test_item_rows_never_exceed_the_cap():
+    # items = a call's distinct experts in order of first appearance, their pairs ascending (brute force below); a token row that names
+    # an expert twice can give an item more pairs than the call has rows: the item keeps its first `cap` pairs and reports `over`
+    import random
+    rnd = random.Random(3)
+    for trial in range(300):
+        R, topk, E = rnd.choice([1, 2, 3, 4, 8]), rnd.choice([1, 2, 6, 10, 16]), rnd.choice([4, 17, 64])
+        if R * topk > 128:
+            continue
+        dup = trial % 3 == 0
+        ex = []
+        for r in range(R):
+            row = [rnd.randrange(E) for _ in range(topk)] if dup else rnd.sample(range(E), min(topk, E)) + [0] * max(0, topk - E)
+            ex += row[:topk]
+        order, pairs = [], {}
+        for p, x in enumerate(ex):
+            if x not in pairs:
+                order.append(x); pairs[x] = []
+            pairs[x].append(p)
+        got = _wave_items(ex, cap=R)
+        assert [g[0] for g in got[:-1]] == order and got[-1][0] == -1
+        for eg, rows, n, over in got[:-1]:
+            assert rows == pairs[eg][:R] and n == min(len(pairs[eg]), R) and over == (len(pairs[eg]) > R)
+            if not dup and topk <= E:
+                assert not over and n == len(pairs[eg])                       # valid routes: never capped
