@@ -173,8 +173,10 @@ SPARK_API int spark_mxfp4_moe_x(const void* x, const void* xs, int R, const int6
  * inside ws (out row pairmap[r * topk + k] belongs to token row r, slot k), valid after ds41_moe_mx_ex(skip_combine = 1).
  * ds41_moe_mx_col_passes: the reference caps the per-pair output at 512 MiB and runs down + combine in 2 or 4 column passes beyond
  * (engine-rs/shim/ds41_mx.cu:1416-1425); the same rule here (prefill-sized calls; no skip_combine with more than one pass).
- * ds41_moe_mx_pair_b16: always 0 (the reference's bf16 per-pair output is an environment switch that is off by default,
- * ds41_mx.cu:1243-1255): the per-pair outputs are fp32.
+ * ds41_moe_mx_pair_b16: 1 when the call's per-pair outputs are bf16: with DS41_MOE_PAIR_BF16=1 in the environment (off by default,
+ * as in the reference, ds41_mx.cu:1243-1255) calls of more than 64 rows keep every pair's down output as the bf16 rounding of its
+ * binary32 sum (half the bytes the down product writes and the sum over the pairs reads); the sums over the pairs stay binary32 in
+ * slot order.  ds41_moe_mx_ws_ptrs then hands out uint16 [P, H] behind its float** argument.
  * ds41_moe_gr16_max: accepted and ignored.  In the reference it moves the row count at which 16-row items give way to 32-row
  * items; here one kernel family serves every row count and a row's bits never depend on the rows around it. */
 SPARK_API void ds41_moe_mx_set_s2(int on);
@@ -312,6 +314,8 @@ SPARK_API void spark_debug_gemv_rows(int v);
 SPARK_API void spark_debug_fp8q_rowmajor(int on);
 /* 256-wide chunks of a wave's K span in that kernel: 1, 2 or 4, 0 = chosen by the shape (a value that does not fit K is ignored) */
 SPARK_API void spark_debug_rm_span(int ch);
+/* the bf16 per-pair outputs of the ds41_* prefill calls: 1 / 0 = on / off, negative = as DS41_MOE_PAIR_BF16 in the environment says */
+SPARK_API void spark_debug_mx_pair_b16(int on);
 /* the cap on the per-pair output buffer of the ds41_* prefill calls in bytes (0 = back to DS41_MOE_OUT_MB or 512 MiB) */
 SPARK_API void spark_debug_mx_out_cap(size_t bytes);
 /* Opt-in check of every expert call's routes on the host before anything is launched (for bringing up an integration): on with 1

@@ -575,6 +575,10 @@ __global__ __launch_bounds__(64 * FW, 4) void fused_kernel(const FArgs a)
     }
     asm volatile("" :: "v"(warm));                         // the warming load is complete before the wave ends
     TRACE(7);
+#ifdef SPK_EXL3_TRACE
+    // where the block ran: XCC_ID (register 20) and HW_ID (register 4: CU, shader array, shader engine)
+    if (a.trace && tid == 0) a.trace[(int64_t)bid * 16 + 8] = ((long long)(__builtin_amdgcn_s_getreg((31 << 11) | 20) & 0xf) << 32) | (uint32_t)__builtin_amdgcn_s_getreg((31 << 11) | 4);
+#endif
 }
 
 // every exchanged word EMPTY, the error flag clear

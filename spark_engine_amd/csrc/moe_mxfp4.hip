@@ -787,8 +787,11 @@ constexpr size_t UP_GEMM_LDS = (size_t)2 * GT_ROWS * GT_XB;
 constexpr int GT_COLS = 256;           // output columns of a down-projection block: two 16-column tiles per wave
 template <int LAYOUT, bool GEN>
 __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __restrict__ hq, const uint8_t* __restrict__ hs, WMat w2, int H, int I,
-                                                           const int* __restrict__ G, const Item* __restrict__ items, float* __restrict__ out, int col0, int ldo)
+                                                           const int* __restrict__ G, const Item* __restrict__ items, float* __restrict__ out, int col0, int ldo,
+                                                           int ob16)
 {
+    // ob16: the pairs' outputs are stored as bf16 (the binary32 sums rounded to nearest even; reference engine-rs/shim/ds41_mx.cu:1245-1255,
+    // DS41_MOE_PAIR_BF16): out is then uint16 [P, ldo]
     // col0 / ldo: this launch covers output columns [col0, col0 + ldo) and out has ldo columns per row (a column pass of a call
     // whose per-pair outputs would not fit the cap on that buffer; one pass: col0 = 0, ldo = H)
     __shared__ __align__(16) unsigned char xl[2][GT_ROWS * GT_XS];
@@ -867,10 +870,16 @@ __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __rest
         const int row = rt * 16 + c;
         if (row < it.n) {
 #pragma unroll
-            for (int m = 0; m < 2; ++m)
+            for (int m = 0; m < 2; ++m) {
                 // written once, read once by the sum over the pairs: a streaming store leaves the caches to the weight stream
-                st_stream16(out + (int64_t)(it.off + row) * ldo + (n0 - col0) + 16 * m + 4 * rg,
-                            make_uint4(__float_as_uint(tot[m][rt][0]), __float_as_uint(tot[m][rt][1]), __float_as_uint(tot[m][rt][2]), __float_as_uint(tot[m][rt][3])));
+                if (ob16)
+                    *(uint2*)((uint16_t*)out + (int64_t)(it.off + row) * ldo + (n0 - col0) + 16 * m + 4 * rg) =
+                        make_uint2((uint32_t)f32_to_bf16(tot[m][rt][0]) | ((uint32_t)f32_to_bf16(tot[m][rt][1]) << 16),
+                                   (uint32_t)f32_to_bf16(tot[m][rt][2]) | ((uint32_t)f32_to_bf16(tot[m][rt][3]) << 16));
+                else
+                    st_stream16(out + (int64_t)(it.off + row) * ldo + (n0 - col0) + 16 * m + 4 * rg,
+                                make_uint4(__float_as_uint(tot[m][rt][0]), __float_as_uint(tot[m][rt][1]), __float_as_uint(tot[m][rt][2]), __float_as_uint(tot[m][rt][3])));
+            }
         }
     }
 }
@@ -878,24 +887,27 @@ __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __rest
 // y[r] = (add[r] + sum of the shared experts' outputs) + (sum_k routed out[pairmap[r, k]], k ascending)
 // reference ds41_mx.cu:302-317
 __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ out, const int* __restrict__ pairmap, const float* __restrict__ add,
-                                                      float* __restrict__ y, int nr, int H, int topk, int n_shared, int col0, int ldo, int obf16)
+                                                      float* __restrict__ y, int nr, int H, int topk, int n_shared, int col0, int ldo, int obf16, int pb16)
 {
-    // columns [col0, col0 + ldo) of y; out has ldo columns per row (one pass: col0 = 0, ldo = H)
+    // columns [col0, col0 + ldo) of y; out has ldo columns per row (one pass: col0 = 0, ldo = H); pb16: the pairs' outputs are bf16
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int h4 = ldo >> 2;
     if (i >= (int64_t)nr * h4) return;
     const int r = (int)(i / h4), col = (int)(i % h4) * 4, TT = topk + n_shared;
     float4 acc = add ? *(const float4*)(add + (int64_t)r * H + col0 + col) : make_float4(0.f, 0.f, 0.f, 0.f);
     // the pairs' outputs are read once: streaming loads
-    for (int k = topk; k < TT; ++k) {
-        const uint4 v = ld_stream16(out + (int64_t)pairmap[r * TT + k] * ldo + col);
-        acc.x += __uint_as_float(v.x); acc.y += __uint_as_float(v.y); acc.z += __uint_as_float(v.z); acc.w += __uint_as_float(v.w);
-    }
+    auto pair4 = [&](int k) {
+        const int64_t o = (int64_t)pairmap[r * TT + k] * ldo + col;
+        if (pb16) {
+            const uint2 v = *(const uint2*)((const uint16_t*)out + o);
+            return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+        }
+        const uint4 v = ld_stream16(out + o);
+        return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+    };
+    for (int k = topk; k < TT; ++k) { const float4 v = pair4(k); acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w; }
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int k = 0; k < topk; ++k) {
-        const uint4 v = ld_stream16(out + (int64_t)pairmap[r * TT + k] * ldo + col);
-        s.x += __uint_as_float(v.x); s.y += __uint_as_float(v.y); s.z += __uint_as_float(v.z); s.w += __uint_as_float(v.w);
-    }
+    for (int k = 0; k < topk; ++k) { const float4 v = pair4(k); s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w; }
     acc.x += s.x; acc.y += s.y; acc.z += s.z; acc.w += s.w;
     if (obf16) *(uint2*)((uint16_t*)y + (int64_t)r * H + col0 + col) = make_uint2((uint32_t)f32_to_bf16(acc.x) | ((uint32_t)f32_to_bf16(acc.y) << 16),
                                                                                    (uint32_t)f32_to_bf16(acc.z) | ((uint32_t)f32_to_bf16(acc.w) << 16));
@@ -973,9 +985,10 @@ inline WsLayout ws_layout(int R, int H, int I, int TT, int ET, int np = 1)
 template <int LAYOUT>
 int moe_launch(const uint8_t* xq, const uint8_t* xs, int R, const int64_t* idx, const float* rw, const uint8_t* w1, const uint8_t* s1, const uint8_t* w3,
                const uint8_t* s3, const uint8_t* w2, const uint8_t* s2, int H, int I, int topk, int E, int n_shared, const float* add, float* y, void* ws,
-               int skip_combine, hipStream_t st, int np = 1, int obf16 = 0)
+               int skip_combine, hipStream_t st, int np = 1, int obf16 = 0, int pb16 = 0)
 {
     const bool gemm = gemm_ok(LAYOUT, R, H, I);
+    if (pb16 && !gemm) return 1;                              // bf16 pair outputs belong to the grouped GEMM
     if (np > 1 && (!gemm || skip_combine)) return 1;          // column passes belong to the grouped GEMM and sum as they go
     const int TT = topk + n_shared, ET = E + n_shared, GR = gr_of(R, gemm), Gm = gmax_of(R, TT, ET, gemm);
     const WsLayout l = ws_layout(R, H, I, TT, ET, np);
@@ -1013,9 +1026,9 @@ int moe_launch(const uint8_t* xq, const uint8_t* xs, int R, const int64_t* idx, 
             for (int ps = 0; ps < np; ++ps) {
                 // a pass = the down product of hn output columns, then (with more than one pass) their weighted sum, before the next
                 // pass writes over the buffer; every output's products and sums are those of the one-pass call
-                if (gend) down_gemm_kernel<LAYOUT, true><<<dim3(hn / GT_COLS, Gm), 512, 0, st>>>(hq, hs, m2, H, I, G, items, out, ps * hn, hn);
-                else down_gemm_kernel<LAYOUT, false><<<dim3(hn / GT_COLS, Gm), 512, 0, st>>>(hq, hs, m2, H, I, G, items, out, ps * hn, hn);
-                if (np > 1) combine_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(out, pairmap, add, y, R, H, topk, n_shared, ps * hn, hn, obf16);
+                if (gend) down_gemm_kernel<LAYOUT, true><<<dim3(hn / GT_COLS, Gm), 512, 0, st>>>(hq, hs, m2, H, I, G, items, out, ps * hn, hn, pb16);
+                else down_gemm_kernel<LAYOUT, false><<<dim3(hn / GT_COLS, Gm), 512, 0, st>>>(hq, hs, m2, H, I, G, items, out, ps * hn, hn, pb16);
+                if (np > 1) combine_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(out, pairmap, add, y, R, H, topk, n_shared, ps * hn, hn, obf16, pb16);
             }
             if (np > 1) return launch_status();
         }
@@ -1028,7 +1041,7 @@ int moe_launch(const uint8_t* xq, const uint8_t* xs, int R, const int64_t* idx, 
     }
     if (!skip_combine) {
         const int64_t n4 = (int64_t)R * (H / 4);
-        combine_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(out, pairmap, add, y, R, H, topk, n_shared, 0, H, obf16);
+        combine_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(out, pairmap, add, y, R, H, topk, n_shared, 0, H, obf16, pb16);
     }
     return launch_status();
 }
@@ -1214,7 +1227,22 @@ SPARK_API void spark_debug_mx_out_cap(size_t bytes) { g_out_cap = bytes; }
 // diagnostics: the most rows the single launch takes where the grouped GEMM could take the call too (negative: the rule per layout)
 SPARK_API void spark_debug_mx_fused_rows(int rows) { g_fused_rows = rows < 0 ? -1 : rows > 8 ? 8 : rows; }
 SPARK_API int ds41_moe_mx_col_passes(int R, int topk, int E) { (void)E; return R < 1 || topk < 1 ? 1 : ds41_rule_passes(R, topk); }
-SPARK_API int ds41_moe_mx_pair_b16(int, int, int) { return 0; }   // the reference's bf16 per-pair output is an environment switch, off by default
+namespace {
+int g_pair_b16 = -1;                   // -1 = not decided yet (DS41_MOE_PAIR_BF16 in the environment decides at the first call), 0 off, 1 on
+// reference ds41_mx.cu:1245-1255: with DS41_MOE_PAIR_BF16=1 (off by default there and here) the prefill-sized calls (more than 64
+// rows, the grouped GEMM) keep every pair's down output as bf16 - the binary32 sum rounded once - instead of binary32: half the bytes
+// the down product writes and the sum over the pairs reads; the sums over the pairs stay binary32 in the same order
+bool pair_b16_on(int R, int I)
+{
+    if (g_pair_b16 < 0) { const char* e = std::getenv("DS41_MOE_PAIR_BF16"); g_pair_b16 = e && e[0] == '1' ? 1 : 0; }
+    return g_pair_b16 == 1 && R > 64 && gemm_ok(L_MX8, R, DS41_H, I);
+}
+}  // namespace
+// diagnostics: 1 / 0 switch the bf16 pair outputs on / off, negative = as the environment says (read again at the next call)
+SPARK_API void spark_debug_mx_pair_b16(int on) { g_pair_b16 = on < 0 ? -1 : on ? 1 : 0; }
+// whether a call's pair outputs (ds41_moe_mx_ws_ptrs) are bf16; the intermediate width does not enter the reference's signature:
+// answered for widths the grouped GEMM takes (every width the reference uses)
+SPARK_API int ds41_moe_mx_pair_b16(int R, int topk, int E) { (void)topk; (void)E; return pair_b16_on(R, 2048) ? 1 : 0; }
 SPARK_API size_t ds41_moe_mx_ws_bytes(int R, int I, int topk, int E) { return ds41_ws_total(R, I, topk, E); }
 SPARK_API size_t ds41_moe_ws_bytes(int R, int I, int topk, int E)
 {
@@ -1232,12 +1260,13 @@ SPARK_API int ds41_moe_mx_ex(const void* xq, const void* xs, int R, const int64_
     // decode sizes: the whole layer in one launch, straight from the reference's tile layout (same bits as the kernels below)
     if (!skip_combine && mx_fused_ok(R, DS41_H, I, topk, E, 0) && !gemm_ok(L_MX8, R, DS41_H, I))
         return mx_fused_launch(xq, xs, R, idx, rw, w1, s1, w3, s3, w2, s2, g_s2 ? L_MX8S2 : L_MX8, DS41_H, I, topk, E, 0, add, y, ws, 0, st);
-    const int np = ds41_passes(R, I, topk);
+    const int np = ds41_passes(R, I, topk), pb = pair_b16_on(R, I) ? 1 : 0;
     if (g_s2)                                                  // s1 / s3 / s2 are 2-bit coded scale blobs
         return moe_launch<L_MX8S2>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3,
-                                   (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, DS41_H, I, topk, E, 0, add, y, ds41_region(ws, I, topk, E), skip_combine, st, np);
+                                   (const uint8_t*)s3, (const uint8_t*)w2, (const uint8_t*)s2, DS41_H, I, topk, E, 0, add, y, ds41_region(ws, I, topk, E), skip_combine, st, np,
+                                   0, pb);
     return moe_launch<L_MX8>((const uint8_t*)xq, (const uint8_t*)xs, R, idx, rw, (const uint8_t*)w1, (const uint8_t*)s1, (const uint8_t*)w3, (const uint8_t*)s3,
-                             (const uint8_t*)w2, (const uint8_t*)s2, DS41_H, I, topk, E, 0, add, y, ds41_region(ws, I, topk, E), skip_combine, st, np);
+                             (const uint8_t*)w2, (const uint8_t*)s2, DS41_H, I, topk, E, 0, add, y, ds41_region(ws, I, topk, E), skip_combine, st, np, 0, pb);
 }
 SPARK_API int ds41_moe_mx(const void* xq, const void* xs, int R, const int64_t* idx, const float* rw, const void* w1, const void* s1, const void* w3,
                           const void* s3, const void* w2, const void* s2, int I, const float* add, float* y, void* ws, int topk, int E, hipStream_t st)
@@ -1253,7 +1282,7 @@ SPARK_API int ds41_moe_mx_combine_rows(void* ws, int R, int I, int topk, int E, 
     const float* out = (const float*)(base + l.out);
     const int64_t n4 = (int64_t)nr * (DS41_H / 4);
     combine_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(out, pairmap + (int64_t)r0 * topk, add ? add + (int64_t)r0 * DS41_H : nullptr,
-                                                                 y + (int64_t)r0 * DS41_H, nr, DS41_H, topk, 0, 0, DS41_H, 0);
+                                                                 y + (int64_t)r0 * DS41_H, nr, DS41_H, topk, 0, 0, DS41_H, 0, pair_b16_on(R, I) ? 1 : 0);
     return launch_status();
 }
 SPARK_API int ds41_moe_mx_combine(void* ws, int R, int I, int topk, int E, const float* add, float* y, hipStream_t st)

@@ -90,6 +90,7 @@ SIGNATURES = {
     "spark_moe_ws_status": (i32, [vp, vp]), "spark_exl3_moe_static_status": (i32, [vp]),
     "spark_moe_ws_release": (None, [vp]),
     # diagnostics
+    "spark_debug_mx_pair_b16": (None, [i32]),
     "spark_debug_stream_read": (i32, [vp, sz, vp, vp]),
     "spark_debug_mx_ws_h": (i32, [vp, i32, i32, i32, i32, i32, i32, vp, vp, vp]),
     "spark_debug_exl3_local": (None, [i32]), "spark_debug_mx_local": (None, [i32]), "spark_debug_exl3_twa": (None, [i32]),

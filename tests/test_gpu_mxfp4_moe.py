@@ -348,3 +348,46 @@ def test_ds41_column_passes_under_a_small_cap(ops, oracle):
                 ops.ds41_moe_mx(xq, xs, dev(idx), dev(rw), w, I, add=dev(add), ws=wsb, skip_combine=True)
     finally:
         L.spark_debug_mx_out_cap(0)
+
+
+def test_ds41_bf16_pair_outputs_switch(ops, oracle):
+    # reference ds41_mx.cu:1245-1255 (DS41_MOE_PAIR_BF16, off by default): calls of more than 64 rows keep every pair's down output as
+    # bf16; the buffer ds41_moe_mx_ws_ptrs hands out then holds the bf16 rounding of what the binary32 form holds, and the sum over the
+    # pairs is the binary32 sum of those in slot order
+    import ctypes as C
+    g = synth.rng(219)
+    R, H, I, E, topk = 70, 5120, 512, 5, 2
+    ws, x, idx, rw = _case(g, R, H, I, E, topk, 0, smin=119)
+    add = g.standard_normal((R, H)).astype(np.float32)
+    w = _ds41_weights(ops, ws)
+    xq, xs = ops.act_quant_fp8(dev_bf16(x))
+    L = ops._lib()
+    assert L.ds41_moe_mx_pair_b16(R, topk, E) == 0
+    y32, wsb32 = ops.ds41_moe_mx(xq, xs, dev(idx), dev(rw), w, I, add=dev(add), skip_combine=True)
+    po, pm = C.c_void_p(), C.c_void_p()
+    assert L.ds41_moe_mx_ws_ptrs(C.c_void_p(wsb32.data_ptr()), R, I, topk, E, C.byref(po), C.byref(pm)) == 0
+    torch.cuda.synchronize()
+    P = R * topk
+    o32 = wsb32[po.value - wsb32.data_ptr():po.value - wsb32.data_ptr() + 4 * P * H].view(torch.float32).view(P, H).clone()
+    pmap32 = wsb32[pm.value - wsb32.data_ptr():pm.value - wsb32.data_ptr() + 4 * P].view(torch.int32).clone()
+    L.spark_debug_mx_pair_b16(1)
+    try:
+        assert L.ds41_moe_mx_pair_b16(R, topk, E) == 1 and L.ds41_moe_mx_pair_b16(64, topk, E) == 0
+        y16, wsb16 = ops.ds41_moe_mx(xq, xs, dev(idx), dev(rw), w, I, add=dev(add))
+        assert L.ds41_moe_mx_ws_ptrs(C.c_void_p(wsb16.data_ptr()), R, I, topk, E, C.byref(po), C.byref(pm)) == 0
+        torch.cuda.synchronize()
+        o16 = wsb16[po.value - wsb16.data_ptr():po.value - wsb16.data_ptr() + 2 * P * H].view(torch.bfloat16).view(P, H)
+        pmap16 = wsb16[pm.value - wsb16.data_ptr():pm.value - wsb16.data_ptr() + 4 * P].view(torch.int32)
+        # (which compact row a pair gets may differ from call to call - the grouping hands rows out with atomics -: compare pair by pair)
+        assert torch.equal(o16[pmap16.long()], o32[pmap32.long()].to(torch.bfloat16))
+        acc = torch.zeros(R, H, dtype=torch.float32, device=DEV)
+        for k in range(topk):
+            acc = acc + o16.float()[pmap16.view(R, topk)[:, k].long()]
+        assert torch.equal(y16, dev(add) + acc)                         # add + (the pairs in slot order), binary32
+        assert rel_l2(host(y16), oracle.mxfp4_moe(x, idx, rw, *ws, add=add)) <= 4e-3      # the bf16 rounding of the pairs: the reference's class L1
+        small, _ = ops.ds41_moe_mx(xq[:40], xs[:40], dev(idx[:40]), dev(rw[:40]), w, I, add=dev(add[:40]))
+    finally:
+        L.spark_debug_mx_pair_b16(0)
+    plain, _ = ops.ds41_moe_mx(xq[:40], xs[:40], dev(idx[:40]), dev(rw[:40]), w, I, add=dev(add[:40]))
+    assert torch.equal(small, plain)                                    # calls of up to 64 rows are not touched by the switch
+    L.spark_debug_mx_pair_b16(-1)
