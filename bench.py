@@ -802,15 +802,15 @@ def main():
         todo += [(lambda R=R, N=N, K=K: Fp8DensePacked(torch, ops, R, INST, N, K), f"{c} batch{R}") for (c, N, K) in (("c4ap", 7168, 4096), ("c4bp", 4096, 7168)) for R in (1, 4)]
         todo += [(lambda: Mxfp4Prefill(torch, ops, 2048, 4), "c5 batch2048"), (lambda: Exl3Prefill(torch, ops, 2048, 4), "c2p batch2048")]
         # the reference model's dense projections (not a configuration: the callers either side of the expert layer)
-        todo += [(lambda N=N, K=K, R=R: Fp8MxProjection(torch, ops, R, INST, N, K), None) for (N, K) in ((12288, 1280), (5120, 3072), (1280, 5120)) for R in (1, 8)]
-        todo += [(lambda R=R: GlmFp8Dense(torch, ops, R, INST, 4096, 4096), None) for R in (1, 4)]
+        todo += [(lambda N=N, K=K, R=R: Fp8MxProjection(torch, ops, R, INST, N, K), f"{c} batch{R}") for (c, N, K) in (("p1", 12288, 1280), ("p2", 5120, 3072), ("p3", 1280, 5120)) for R in (1, 8)]
+        todo += [(lambda R=R: GlmFp8Dense(torch, ops, R, INST, 4096, 4096), f"g8 batch{R}") for R in (1, 4)]
         # the sizes the reference's own kernels are compiled for, through spark_* and through the reference-named entry points
         # (a caller that changes nothing: workspace contents undefined, no *_ws_init; and with the one added *_ws_init call)
-        todo += [(mk, None) for mk in (
-                 lambda: Exl3LayerQwen(torch, ops, 1, INST), lambda: QwenReferenceEntry(torch, ops, 1, INST, prepared=False),
-                 lambda: QwenReferenceEntry(torch, ops, 1, INST, prepared=True), lambda: Exl3LayerGlm(torch, ops, 1, INST),
-                 lambda: Mxfp4LayerWide(torch, ops, 1, INST), lambda: Ds41ReferenceEntry(torch, ops, 1, INST, prepared=False),
-                 lambda: Ds41ReferenceEntry(torch, ops, 1, INST, prepared=True), lambda: Ds41ReferenceEntryRank(torch, ops, 1, INST, prepared=True))]
+        todo += [(lambda: Exl3LayerQwen(torch, ops, 1, INST), "c2q batch1"), (lambda: QwenReferenceEntry(torch, ops, 1, INST, prepared=False), "c2ref batch1"),
+                 (lambda: QwenReferenceEntry(torch, ops, 1, INST, prepared=True), "c2refp batch1"), (lambda: Exl3LayerGlm(torch, ops, 1, INST), "c2g batch1"),
+                 (lambda: Mxfp4LayerWide(torch, ops, 1, INST), "c3w batch1"), (lambda: Ds41ReferenceEntry(torch, ops, 1, INST, prepared=False), "c3ref batch1"),
+                 (lambda: Ds41ReferenceEntry(torch, ops, 1, INST, prepared=True), "c3refp batch1"),
+                 (lambda: Ds41ReferenceEntryRank(torch, ops, 1, INST, prepared=True), "c3rank batch1")]
         for mk, tag in todo:
             w2 = mk()
             ln = line_for(w2, *time_protocol(torch, w2), tag=tag, floor=(torch, ops))

@@ -62,14 +62,15 @@ __global__ __launch_bounds__(64 * T16_WAVES) void fp8_t16_gemv_kernel(const uint
     const int kb0 = wave * T16_SPAN, nb = min(T16_SPAN, nkb - kb0);          // 1 .. T16_SPAN by the launch
     // the span's activations: 16-byte pieces, piece c = lane + 64 u of the MX x (T16_SPAN * 16) pieces of the wave's rows
     uint16_t* xw = t16_x + (size_t)wave * (MX * T16_XLD);
-    // (requested with an instruction the compiler does not move: left to itself it sinks these loads below the weight loads, next to
-    // the LDS writes, where each one waits for the whole weight span; the wait before the writes is written out below)
+    // (left to itself the compiler sinks these loads below the weight loads, next to the LDS writes, where each one waits for the
+    // whole weight span: a scheduling fence keeps them ahead, and the compiler counts the wait before the writes itself - loads
+    // return in issue order, so the writes wait for everything but the 2 * T16_SPAN weight loads)
     v4i xt[2 * MX];
 #pragma unroll
     for (int u = 0; u < 2 * MX; ++u) {
         const int c = lane + 64 * u, r = min(c >> 7, m - 1), col = min(c & 127, nb * 16 - 1) * 8;
         const uint16_t* xp = x + (int64_t)r * xs + kb0 * 128 + col;
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xt[u]) : "v"(xp) : "memory");
+        xt[u] = *(const v4i*)xp;
     }
     // the span's scales, one K block per lane (lanes 0-7): a binary32 factor, or the four E8M0 bytes of the block's steps
     float scv = 0.f;
@@ -77,6 +78,7 @@ __global__ __launch_bounds__(64 * T16_WAVES) void fp8_t16_gemv_kernel(const uint
     if constexpr (E8) scw = ((const uint32_t*)((const uint8_t*)scp + (int64_t)(n0 >> 5) * (k >> 5)))[kb0 + min(lane & 7, nb - 1)];
     else scv = ((const float*)scp)[(int64_t)(n0 >> 7) * nkb + kb0 + min(lane & 7, nb - 1)];
     const uint8_t* wp = wt + ((int64_t)nt * nkb + kb0) * T16_TILE + lane * 16;
+    __builtin_amdgcn_sched_barrier(0);
     // (past a short span's end the last K block is requested again: the same lines, nothing is used)
     uint4 p[T16_SPAN][2];
 #pragma unroll
@@ -84,9 +86,7 @@ __global__ __launch_bounds__(64 * T16_WAVES) void fp8_t16_gemv_kernel(const uint
         const int bb = min(b, nb - 1);
         p[b][0] = ld_stream16(wp + bb * T16_TILE); p[b][1] = ld_stream16(wp + bb * T16_TILE + 1024);
     }
-    // loads return in order: when at most the 2 * T16_SPAN weight loads are outstanding, the activations are here
-    static_assert(2 * T16_SPAN == 16, "the wait below counts the weight loads");
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < 2 * MX; ++u) {
         const int c = lane + 64 * u;
@@ -202,16 +202,16 @@ __global__ __launch_bounds__(64 * rm_waves<CH>()) void fp8_rm_gemv_kernel(const 
         const int c = lane + 64 * u, r = min(c / PR, m - 1), pc = min(c % PR, nb * (PR / SPAN) - 1);
         if constexpr (XMODE == 0) {
             const uint16_t* xp = x + xoff + (int64_t)r * xs + kb0 * 128 + pc * 8;
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xt[u]) : "v"(xp) : "memory");
+            xt[u] = *(const v4i*)xp;
         } else if constexpr (XMODE == 1) {
             const uint8_t* xp = aq + (int64_t)r * k + kb0 * 128 + pc * 16;
             const uint8_t* sp = as_ + (int64_t)r * (k >> 5) + kb0 * 4 + (pc >> 1);          // the scale byte of the piece's block of 32
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xt[u]) : "v"(xp) : "memory");
-            asm volatile("global_load_ubyte %0, %1, off" : "=v"(sb[u]) : "v"(sp) : "memory");
+            xt[u] = *(const v4i*)xp;
+            sb[u] = *sp;
         } else {
             const uint16_t* xp = x + (int64_t)r * xs + kb0 * 128 + pc * 16;
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xt[2 * u]) : "v"(xp) : "memory");
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xt[2 * u + 1]) : "v"(xp + 8) : "memory");
+            xt[2 * u] = *(const v4i*)xp;
+            xt[2 * u + 1] = *(const v4i*)(xp + 8);
         }
     }
     float scv = 0.f;
@@ -221,6 +221,7 @@ __global__ __launch_bounds__(64 * rm_waves<CH>()) void fp8_rm_gemv_kernel(const 
     const uint8_t* wp[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) wp[i] = w + (int64_t)min(n0 + lr + 4 * i, n - 1) * k + kb0 * 128 + lc;
+    __builtin_amdgcn_sched_barrier(0);
     uint4 p[CH][4];
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch) {
@@ -228,10 +229,9 @@ __global__ __launch_bounds__(64 * rm_waves<CH>()) void fp8_rm_gemv_kernel(const 
 #pragma unroll
         for (int i = 0; i < 4; ++i) p[ch][i] = ld_stream16(wp[i] + cc * 256);
     }
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(4 * CH) : "memory");     // everything but the weight loads has arrived
-    // the registers the loads above wrote, as seen after the wait (nothing computed from them is scheduled ahead of it)
-#pragma unroll
-    for (int u = 0; u < (XMODE == 2 ? 2 * NU : NU); ++u) asm volatile("" : "+v"(xt[u]));
+    // The activation and scale loads stay ahead of the weight loads (a wave's loads return in issue order: staging then waits for
+    // everything but the 4 CH weight loads, and the compiler counts that wait itself); nothing moves across the two fences.
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
         const int c = lane + 64 * u;
@@ -240,7 +240,6 @@ __global__ __launch_bounds__(64 * rm_waves<CH>()) void fp8_rm_gemv_kernel(const 
         } else {
             uint32_t cw[4], e;
             if constexpr (XMODE == 1) {
-                asm volatile("" : "+v"(sb[u]));
                 cw[0] = (uint32_t)xt[u].x; cw[1] = (uint32_t)xt[u].y; cw[2] = (uint32_t)xt[u].z; cw[3] = (uint32_t)xt[u].w;
                 e = (uint32_t)sb[u] & 0xffu;
             } else {
