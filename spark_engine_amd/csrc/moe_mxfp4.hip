@@ -476,13 +476,25 @@ template <int LAYOUT, bool GEN> struct ATile {
     const uint8_t* raw;                // MX8S2: the tile's raw scale words when it has them (else null)
     uint32_t base4;                    // MX8S2: the row's base scale in all four bytes
     int steps, g;                      // 128-wide K steps of the matrix (the last K group may hold fewer than four); lane / 16
+    uint32_t lo;                       // T16: the lane's offset inside a step's 1024 code bytes (a quarter of it inside the scale bytes)
     static constexpr bool MXT = LAYOUT == L_MX8 || LAYOUT == L_MX8S2;       // 4 x 4 dword order inside a row's 64 bytes
+    // an address that is the same in every lane, pinned to scalar registers: the compiler then keeps scalar base + lane offset apart
+    // (left alone it folds the lane offset into a 64-bit pointer per lane and stream, and those spill beside the weight ring)
+    typedef const __attribute__((address_space(1))) uint8_t* GPtr;          // (an integer turned pointer must say that it is global memory)
+    __device__ __forceinline__ static GPtr uniform(const uint8_t* p)
+    {
+        uint64_t b = (uint64_t)p;
+        asm volatile("" : "+s"(b));
+        return (GPtr)b;
+    }
     __device__ __forceinline__ ATile(const WMat& m, int64_t row0, int lane)          // row0: first row of the tile in the stacked matrix
     {
         steps = m.K >> 7; g = lane >> 4;
         if constexpr (LAYOUT == L_T16) {
-            const uint8_t* rec = m.w + (row0 >> 4) * (int64_t)((steps + 3) >> 2) * REC;      // a ragged last K group is a whole record, zero filled
-            w = rec + lane * 16; sc = rec + 4096 + lane * 4;
+            // the tile's first record is the same address for the whole wave (row0 is uniform): kept apart from the lane's offset so that
+            // the loads address it as scalar base + 32-bit lane offset (one register a lane instead of a 64-bit pointer per stream)
+            w = m.w + (row0 >> 4) * (int64_t)((steps + 3) >> 2) * REC;      // a ragged last K group is a whole record, zero filled
+            sc = w + 4096; lo = (uint32_t)lane * 16u;
         } else {
             const int64_t row = row0 + (lane & 15), t8 = row >> 3;
             const int r8 = (int)(row & 7);
@@ -501,9 +513,10 @@ template <int LAYOUT, bool GEN> struct ATile {
     // GEN: steps past the matrix (the tail of a ragged last K group) read the last step again: a valid address, multiplied by zeros
     __device__ __forceinline__ v4i codes(int kg, int s) const
     {
-        const uint8_t* p;
-        if constexpr (LAYOUT == L_T16) p = w + (int64_t)kg * REC + s * 1024;
-        else p = w + (int64_t)(GEN ? min(kg * 4 + s, steps - 1) : kg * 4 + s) * 512;
+        if constexpr (LAYOUT == L_T16) {
+            return *(const __attribute__((address_space(1))) v4i*)(uniform(w + (int64_t)kg * REC) + s * 1024 + lo);
+        }
+        const uint8_t* p = w + (int64_t)(GEN ? min(kg * 4 + s, steps - 1) : kg * 4 + s) * 512;
         const uint4 v = *(const uint4*)p;
         return v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
     }
@@ -520,7 +533,7 @@ template <int LAYOUT, bool GEN> struct ATile {
     }
     __device__ __forceinline__ uint32_t scales_raw(int kg) const
     {
-        if constexpr (LAYOUT == L_T16) return *(const uint32_t*)(sc + (int64_t)kg * REC);
+        if constexpr (LAYOUT == L_T16) return *(const __attribute__((address_space(1))) uint32_t*)(uniform(sc + (int64_t)kg * REC) + (lo >> 2));
         else {
             const int step = GEN ? min(kg * 4 + g, steps - 1) : kg * 4 + g;   // this lane fetches the four block scales of step g of the K group
             if constexpr (LAYOUT == L_MX8S2) {
@@ -647,29 +660,33 @@ __device__ __forceinline__ XStageB xb_fetch(const uint8_t* xrow, const uint8_t* 
 }
 __device__ __forceinline__ void xb_put(const XStageB& r, unsigned char* dst)
 {
+    // eight codes (two dwords) at a time: converted and stored before the next eight, so that few registers are live beside the K loop's
     const uint32_t m = r.in ? ~0u : 0u;
-    const XOp o = x_operand(make_uint4(r.x0.x & m, r.x0.y & m, r.x0.z & m, r.x0.w & m), make_uint4(r.x1.x & m, r.x1.y & m, r.x1.z & m, r.x1.w & m), r.sb);
+    const float sc = e8m0_to_f32(r.sb & 0xffu);
+    const uint32_t w[8] = {r.x0.x & m, r.x0.y & m, r.x0.z & m, r.x0.w & m, r.x1.x & m, r.x1.y & m, r.x1.z & m, r.x1.w & m};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) { uint4 v; __builtin_memcpy(&v, &o.b[j], 16); *(uint4*)(dst + 16 * j) = v; }
+    for (int j = 0; j < 4; ++j) {
+        bf2 v[4];
+        v[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j], sc, false); v[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j], sc, true);
+        v[2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j + 1], sc, false); v[3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j + 1], sc, true);
+        uint4 o; __builtin_memcpy(&o, v, 16);
+        *(uint4*)(dst + 16 * j) = o;
+        __builtin_amdgcn_sched_barrier(0);
+    }
 }
 
-template <int LAYOUT, bool GEN>
-__global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, WMat w1, WMat w3, int H, int I, int TT,
-                                                         const int* __restrict__ G, const Item* __restrict__ items, const int* __restrict__ prow,
-                                                         const float* __restrict__ pw, uint8_t* __restrict__ hq, uint8_t* __restrict__ hs)
+// One block of the gate / up GEMM for an item of NRT 16-row tiles.  The kernel below runs the instance of the item's tile count: each
+// instance is a region of its own for the register allocator (one K loop with a run-time tile count put a branch into every step;
+// two K loops sharing their surroundings spilled beside the weight ring).
+template <int LAYOUT, bool GEN, int NRT>
+__device__ __forceinline__ void up_gemm_block(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const WMat& w1, const WMat& w3, int H, int I, int TT,
+                                              const Item it, const int* __restrict__ prow, const float* __restrict__ pw, uint8_t* __restrict__ hq,
+                                              uint8_t* __restrict__ hs, unsigned char* gsm, int* toks, float* wgts, float (*amx)[2][16], unsigned char (*hes)[4])
 {
-    extern __shared__ __align__(16) unsigned char gsm[];  // xl [2][GT_ROWS * GT_XB], then the epilogue's hbuf [GT_ROWS][GT_FEAT + 16] over it
-    __shared__ int toks[GT_ROWS];
-    __shared__ float wgts[GT_ROWS];
-    __shared__ float amx[8][2][16];
-    __shared__ __align__(4) unsigned char hes[GT_ROWS][4];
     unsigned char* const xl = gsm;
-    const Item it = items[blockIdx.y];             // requested together with the item count (entries past it hold anything)
-    if ((int)blockIdx.y >= *G) return;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, rg = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), c = lane & 15, rg = lane >> 4;
     const int f0 = blockIdx.x * GT_FEAT;
     const int steps = H >> 7, nkg = (steps + 3) >> 2;      // the last K group may hold fewer than four steps
-    const int nrt = (it.n + 15) >> 4;
     if (tid < GT_ROWS) {
         const int pos = it.off + min(tid, it.n - 1);
         toks[tid] = prow[pos] / TT;
@@ -693,66 +710,83 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
     xb_put(xf, xdst);
     xf = xb_fetch<GEN>(xrow, xsrow, kg1, sch, H);
     __syncthreads();
-    v4f tot[2][2];
+    v4f tot[2][NRT];
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) tot[m][rt] = v4f{0.f, 0.f, 0.f, 0.f};
-    v4f cur[2][2];
+        for (int rt = 0; rt < NRT; ++rt) tot[m][rt] = v4f{0.f, 0.f, 0.f, 0.f};
     const unsigned char* const bbase = xl + c * GT_XB + 64 * rg;
-    for (int i = 0; i < nkg; ++i) {
-        const KVisit vis = k_visit<GEN, UP_WAVES>(i, nkg);
-        const int buf = i & 1, kn = k_visit<GEN, UP_WAVES>(min(i + 1, nkg - 1), nkg).kg;
-        const uint32_t san0 = t1.scales_raw(kn), san1 = t3.scales_raw(kn);
-        const uint32_t sc0 = ATile<LAYOUT, GEN>::scales_fix(sa[0], lane), sc1 = ATile<LAYOUT, GEN>::scales_fix(sa[1], lane);
-        if (vis.fresh) {
+    // The K loop in two instances, for items of one and of two 16-row tiles: no branch inside a K group, so that the compiler
+    // schedules a K group's 16-byte operand reads, converts and matrix instructions as one block (with a branch around the second
+    // row tile's instructions every read waited for its data right in front of its matrix instruction).
+    {
+        v4f cur[2][NRT];
+        for (int i = 0; i < nkg; ++i) {
+            const KVisit vis = k_visit<GEN, UP_WAVES>(i, nkg);
+            const int buf = i & 1, kn = k_visit<GEN, UP_WAVES>(min(i + 1, nkg - 1), nkg).kg;
+            const uint32_t san0 = t1.scales_raw(kn), san1 = t3.scales_raw(kn);
+            const uint32_t sc0 = ATile<LAYOUT, GEN>::scales_fix(sa[0], lane), sc1 = ATile<LAYOUT, GEN>::scales_fix(sa[1], lane);
+            if (vis.fresh) {
 #pragma unroll
-            for (int m = 0; m < 2; ++m)
+                for (int m = 0; m < 2; ++m)
 #pragma unroll
-                for (int rt = 0; rt < 2; ++rt) cur[m][rt] = v4f{0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-        for (int m = 0; m < 2; ++m)
-#pragma unroll
-            for (int rt = 0; rt < 2; ++rt) asm volatile("" : "+v"(cur[m][rt]));
-        const unsigned char* bp = bbase + buf * (GT_ROWS * GT_XB);
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const v4i a0 = ATile<LAYOUT, GEN>::fix(a[0][s]), a1 = ATile<LAYOUT, GEN>::fix(a[1][s]);
-            const float f0s = e8m0_to_f32((sc0 >> (8 * s)) & 0xffu), f1s = e8m0_to_f32((sc1 >> (8 * s)) & 0xffu);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const bf8v w0 = a_operand((uint32_t)a0[j], f0s), w1v = a_operand((uint32_t)a1[j], f1s);
-                bf8v b0, b1;
-                { const uint4 v = *(const uint4*)(bp + s * 256 + 16 * j); __builtin_memcpy(&b0, &v, 16); }
-                cur[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, b0, cur[0][0], 0, 0, 0);
-                cur[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1v, b0, cur[1][0], 0, 0, 0);
-                if (nrt > 1) {
-                    { const uint4 v = *(const uint4*)(bp + 16 * GT_XB + s * 256 + 16 * j); __builtin_memcpy(&b1, &v, 16); }
-                    cur[0][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, b1, cur[0][1], 0, 0, 0);
-                    cur[1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1v, b1, cur[1][1], 0, 0, 0);
-                }
+                    for (int rt = 0; rt < NRT; ++rt) cur[m][rt] = v4f{0.f, 0.f, 0.f, 0.f};
             }
-            a[0][s] = t1.codes(kn, s);                 // the ring slot is free again: the same step of the next K group
-            a[1][s] = t3.codes(kn, s);
-        }
-        if (vis.last) {
 #pragma unroll
             for (int m = 0; m < 2; ++m)
 #pragma unroll
-                for (int rt = 0; rt < 2; ++rt) tot[m][rt] += cur[m][rt];
+                for (int rt = 0; rt < NRT; ++rt) asm volatile("" : "+v"(cur[m][rt]));
+            const unsigned char* bp = bbase + buf * (GT_ROWS * GT_XB);
+            // B operands one step ahead of their matrix instructions: step t = (s, j) reads the operands of step t + 1 first
+            auto read_b = [&](int t, bf8v (&b)[NRT]) {
+#pragma unroll
+                for (int rt = 0; rt < NRT; ++rt) {
+                    const uint4 v = *(const uint4*)(bp + rt * (16 * GT_XB) + (t >> 2) * 256 + 16 * (t & 3));
+                    __builtin_memcpy(&b[rt], &v, 16);
+                }
+            };
+            constexpr bool AHEAD = NRT == 1 || LAYOUT == L_T16;    // (the tile layouts with two row tiles have no registers left for the second set of operands)
+            bf8v bq[AHEAD ? 2 : 1][NRT];
+            if constexpr (AHEAD) read_b(0, bq[0]);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const v4i a0 = ATile<LAYOUT, GEN>::fix(a[0][s]), a1 = ATile<LAYOUT, GEN>::fix(a[1][s]);
+                const float f0s = e8m0_to_f32((sc0 >> (8 * s)) & 0xffu), f1s = e8m0_to_f32((sc1 >> (8 * s)) & 0xffu);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int t = 4 * s + j;
+                    if constexpr (AHEAD) { if (t < 15) read_b(t + 1, bq[(t + 1) & 1]); }
+                    else read_b(t, bq[0]);                 // requested ahead of the step's converts
+                    __builtin_amdgcn_sched_barrier(0);
+                    const bf8v w0 = a_operand((uint32_t)a0[j], f0s), w1v = a_operand((uint32_t)a1[j], f1s);
+#pragma unroll
+                    for (int rt = 0; rt < NRT; ++rt) {
+                        cur[0][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, bq[AHEAD ? (t & 1) : 0][rt], cur[0][rt], 0, 0, 0);
+                        cur[1][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1v, bq[AHEAD ? (t & 1) : 0][rt], cur[1][rt], 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                a[0][s] = t1.codes(kn, s);                 // the ring slot is free again: the same step of the next K group
+                a[1][s] = t3.codes(kn, s);
+            }
+            if (vis.last) {
+#pragma unroll
+                for (int m = 0; m < 2; ++m)
+#pragma unroll
+                    for (int rt = 0; rt < NRT; ++rt) tot[m][rt] += cur[m][rt];
+            }
+            sa[0] = san0; sa[1] = san1;
+            // the next K group of the rows into the other buffer (nobody reads it before the barrier), the one after into registers
+            xb_put(xf, xdst + (buf ^ 1) * (GT_ROWS * GT_XB));
+            xf = xb_fetch<GEN>(xrow, xsrow, k_visit<GEN, UP_WAVES>(min(i + 2, nkg - 1), nkg).kg, sch, H);
+            __syncthreads();
         }
-        sa[0] = san0; sa[1] = san1;
-        // the next K group of the rows into the other buffer (nobody reads it before the barrier), the one after into registers
-        xb_put(xf, xdst + (buf ^ 1) * (GT_ROWS * GT_XB));
-        xf = xb_fetch<GEN>(xrow, xsrow, k_visit<GEN, UP_WAVES>(min(i + 2, nkg - 1), nkg).kg, sch, H);
-        __syncthreads();
     }
     // ---- SwiGLU * route weight, act_quant per 32 features (this wave's 16 and its neighbour's), 128 code bytes + 4 scales per row
     unsigned char (*hbuf)[GT_FEAT + 16] = (unsigned char (*)[GT_FEAT + 16])gsm;     // the staging buffers are free: the loop ended on a barrier
-    float yv[2][4];
+    float yv[NRT][4];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
+    for (int rt = 0; rt < NRT; ++rt) {
         const float wgt = wgts[rt * 16 + c];
         float am = 0.f;
 #pragma unroll
@@ -768,7 +802,7 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
     }
     __syncthreads();
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
+    for (int rt = 0; rt < NRT; ++rt) {
         const uint32_t e = aq_scale(fmaxf(amx[wave][rt][c], amx[wave ^ 1][rt][c]));
         *(uint32_t*)&hbuf[rt * 16 + c][16 * wave + 4 * rg] = aq_word4(yv[rt][0], yv[rt][1], yv[rt][2], yv[rt][3], e);
         if (rg == 0 && (wave & 1) == 0) hes[rt * 16 + c][wave >> 1] = (unsigned char)e;
@@ -781,6 +815,21 @@ __global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restri
         const int row = tid - 256;
         if (row < it.n) *(uint32_t*)(hs + (int64_t)(it.off + row) * (I >> 5) + (f0 >> 5)) = *(const uint32_t*)hes[row];
     }
+}
+template <int LAYOUT, bool GEN>
+__global__ __launch_bounds__(512, 4) void up_gemm_kernel(const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, WMat w1, WMat w3, int H, int I, int TT,
+                                                         const int* __restrict__ G, const Item* __restrict__ items, const int* __restrict__ prow,
+                                                         const float* __restrict__ pw, uint8_t* __restrict__ hq, uint8_t* __restrict__ hs)
+{
+    extern __shared__ __align__(16) unsigned char gsm[];  // xl [2][GT_ROWS * GT_XB], then the epilogue's hbuf [GT_ROWS][GT_FEAT + 16] over it
+    __shared__ int toks[GT_ROWS];
+    __shared__ float wgts[GT_ROWS];
+    __shared__ float amx[8][2][16];
+    __shared__ __align__(4) unsigned char hes[GT_ROWS][4];
+    const Item it = items[blockIdx.y];             // requested together with the item count (entries past it hold anything)
+    if ((int)blockIdx.y >= *G) return;
+    if (it.n > 16) up_gemm_block<LAYOUT, GEN, 2>(xq, xs, w1, w3, H, I, TT, it, prow, pw, hq, hs, gsm, toks, wgts, amx, hes);
+    else up_gemm_block<LAYOUT, GEN, 1>(xq, xs, w1, w3, H, I, TT, it, prow, pw, hq, hs, gsm, toks, wgts, amx, hes);
 }
 constexpr size_t UP_GEMM_LDS = (size_t)2 * GT_ROWS * GT_XB;
 
@@ -798,7 +847,7 @@ __global__ __launch_bounds__(512, 4) void down_gemm_kernel(const uint8_t* __rest
     __shared__ __align__(16) unsigned char xsl[2][GT_ROWS * 16];
     const Item it = items[blockIdx.y];             // requested together with the item count (entries past it hold anything)
     if ((int)blockIdx.y >= *G) return;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, rg = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), c = lane & 15, rg = lane >> 4;
     const int n0 = col0 + blockIdx.x * GT_COLS + 32 * wave;
     const int steps = I >> 7, nkg = (steps + 3) >> 2;      // the last K group may hold fewer than four steps
     const int nrt = (it.n + 15) >> 4;
