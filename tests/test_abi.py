@@ -65,3 +65,14 @@ def test_load_types_every_symbol():
     handle = lib.load()
     for name in lib.SIGNATURES:
         assert getattr(handle, name).argtypes is not None
+
+
+def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
+    # the product has no CPU path: without the built shared object every operator raises, and says how to build it
+    from spark_engine_amd import lib, ops
+    monkeypatch.setattr(lib, "_lib", None)
+    monkeypatch.setattr(lib, "SO", tmp_path / "libspark_shim_hip.so")
+    with pytest.raises(RuntimeError, match="is missing"):
+        lib.load()
+    with pytest.raises(RuntimeError, match="is missing"):
+        ops._lib()
