@@ -82,3 +82,40 @@ def test_exl3_layer_random_shapes(ops, oracle, R, H, I, E, topk, cbk, act):
     if R <= 8:                                                         # within the single launch a row's bits do not depend on the batch
         o1 = host(ops.exl3_moe(dev_bf16(xb[:1]), dev(idx[:1]), dev(w[:1]), table, H, I, cbk, act))
         assert np.array_equal(o1[0], out[0])
+
+
+def _ds41_cases(n, seed):
+    g = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        I = int(g.choice([128, 256, 512, 640, 768, 1024, 1536, 2048, 2304]))
+        E = int(g.integers(2, 12))
+        topk = int(g.integers(1, min(E, 6) + 1))
+        R = int(g.choice([1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 40, 70]))
+        if I > 1024:
+            R = min(R, 17)
+        out.append((R, I, E, topk))
+    return out
+
+
+@pytest.mark.parametrize("R,I,E,topk", _ds41_cases(10, 9003))
+def test_ds41_entry_points_random_shapes(ops, oracle, R, I, E, topk):
+    # the reference-named entry points (hidden width 5120) on the reference's two tile layouts, raw scale bytes: against the oracle, and
+    # bit for bit against the record layout (every path and layout gives a row the same bits)
+    H = 5120
+    g = synth.rng(R * 13 + I + E)
+    ws = synth.mxfp4_experts(g, E, H, I, 119)
+    x = synth.randn_bf16(g, (R, H))
+    idx = np.stack([g.permutation(E)[:topk] for _ in range(R)]).astype(np.int64)
+    rw = g.uniform(0.1, 1.0, (R, topk)).astype(np.float32)
+    add = g.standard_normal((R, H)).astype(np.float32)
+    ref = oracle.mxfp4_moe(x, idx, rw, *ws, add=add)
+    d = [dev(a) for a in ws]
+    p1, ps1 = ops.moe_pack(d[0], d[1]); p3, ps3 = ops.moe_pack(d[2], d[3]); p2, ps2 = ops.moe_pack(d[4], d[5])
+    xq, xs = ops.act_quant_fp8(dev_bf16(x))
+    y_mx, _ = ops.ds41_moe_mx(xq, xs, dev(idx), dev(rw), (ops.moe_pack_mx(p1), ps1, ops.moe_pack_mx(p3), ps3, ops.moe_pack_mx(p2), ps2), I, add=dev(add))
+    assert rel_l2(host(y_mx), ref) <= TOL, rel_l2(host(y_mx), ref)
+    y_p8 = ops.ds41_moe(ops.act_quant(dev_bf16(x)), dev(idx), dev(rw), (p1, ps1, p3, ps3, p2, ps2), I, add=dev(add))
+    assert np.array_equal(host(y_p8), host(y_mx))
+    y_rec = host(ops.mxfp4_moe(dev_bf16(x), dev(idx), dev(rw), ops.Mxfp4Experts(*d), add=dev(add)))
+    assert np.array_equal(y_rec, host(y_mx))
