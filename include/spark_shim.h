@@ -100,6 +100,10 @@ SPARK_API int spark_sigmoid_route(const float* logits, const float* bias, int64_
 SPARK_API int glm53_router_split(void);
 SPARK_API int glm53_router_fused_cuda(const float* h, const void* w, int w_bf16, const float* bias, float* partial, long long* ids,
                                       float* weights, int rows, int experts, int k, float scaling, hipStream_t st);
+/* The same, and wh [rows, 8] binary16 receives the round-to-nearest-even copy of the weights (what glm_moe_experts takes as w).
+ * Replaces engine-rs/shim/dataflow.cu:549-574 (GLM53_ROUTER_HALF_W=1; Rust caller engine-rs/src/moe.rs:66-67). */
+SPARK_API int glm53_router_fused_h_cuda(const float* h, const void* w, int w_bf16, const float* bias, float* partial, long long* ids,
+                                        float* weights, void* wh, int rows, int experts, int k, float scaling, hipStream_t st);
 
 /* ---------------------------------------------------------------- dense quantised GEMVs (m <= 8 rows) ----------------------- */
 

@@ -212,13 +212,19 @@ __global__ __launch_bounds__(512) void glm_logits_kernel(const float* __restrict
     }
 }
 __global__ __launch_bounds__(256) void glm_select_kernel(const float* __restrict__ partial, const float* __restrict__ bias, long long* __restrict__ ids,
-                                                         float* __restrict__ weights, int experts, int K, float scaling)
+                                                         float* weights, int experts, int K, float scaling, uint16_t* __restrict__ wh)
 {
+    // wh (may be null): the binary16 copy of the row's weights, round to nearest even, for the expert entry points that take them so
     __shared__ float lg[320];
     const int r = blockIdx.x;
     for (int e = threadIdx.x; e < experts; e += 256) lg[e] = partial[((int64_t)r * experts + e) * 2] + partial[((int64_t)r * experts + e) * 2 + 1];
     __syncthreads();
     route_block<2, 2, long long>(lg, bias, ids + (int64_t)r * K, weights + (int64_t)r * K, experts, K, scaling);
+    if (wh) {
+        __threadfence_block();
+        __syncthreads();                                   // the row's weights are written: the same values, rounded once
+        if ((int)threadIdx.x < K) wh[(int64_t)r * K + threadIdx.x] = f32_to_f16_bits(__hip_atomic_load(weights + (int64_t)r * K + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
+    }
 }
 
 }  // namespace
@@ -266,6 +272,17 @@ SPARK_API int glm53_router_fused_cuda(const float* h, const void* w, int w_bf16,
     if (rows < 1 || rows > 32 || experts < 8 || experts > 320 || k % 256) return (int)hipErrorInvalidValue;
     if (w_bf16) glm_logits_kernel<uint16_t><<<experts, 512, 0, st>>>(h, (const uint16_t*)w, partial, rows, experts, k);
     else glm_logits_kernel<float><<<experts, 512, 0, st>>>(h, (const float*)w, partial, rows, experts, k);
-    glm_select_kernel<<<rows, 256, 0, st>>>(partial, bias, ids, weights, experts, 8, scaling);
+    glm_select_kernel<<<rows, 256, 0, st>>>(partial, bias, ids, weights, experts, 8, scaling, nullptr);
+    return launch_status();
+}
+// reference dataflow.cu:549-574 (GLM53_ROUTER_HALF_W=1): the same, and wh [rows, 8] receives the binary16 rounding of the weights
+// that glm_moe_experts takes (the reference otherwise converts them in a launch of its own)
+SPARK_API int glm53_router_fused_h_cuda(const float* h, const void* w, int w_bf16, const float* bias, float* partial, long long* ids, float* weights,
+                                        void* wh, int rows, int experts, int k, float scaling, hipStream_t st)
+{
+    if (rows < 1 || rows > 32 || experts < 8 || experts > 320 || k % 256 || !wh) return (int)hipErrorInvalidValue;
+    if (w_bf16) glm_logits_kernel<uint16_t><<<experts, 512, 0, st>>>(h, (const uint16_t*)w, partial, rows, experts, k);
+    else glm_logits_kernel<float><<<experts, 512, 0, st>>>(h, (const float*)w, partial, rows, experts, k);
+    glm_select_kernel<<<rows, 256, 0, st>>>(partial, bias, ids, weights, experts, 8, scaling, (uint16_t*)wh);
     return launch_status();
 }

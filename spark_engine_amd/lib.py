@@ -41,6 +41,7 @@ SIGNATURES = {
     "spark_sigmoid_route": (i32, [vp, vp, vp, vp, i32, i32, i32, f32, vp]),
     "glm53_router_split": (i32, []),
     "glm53_router_fused_cuda": (i32, [vp, vp, i32, vp, vp, vp, vp, i32, i32, i32, f32, vp]),
+    "glm53_router_fused_h_cuda": (i32, [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, f32, vp]),
     # dense GEMVs
     "ds41_mxfp4_gemv": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
     "ds41_fp8_gemv": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),

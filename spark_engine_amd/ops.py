@@ -259,13 +259,19 @@ def sigmoid_route(logits, bias, k, scaling):
     return idx, w
 
 
-def glm_router_fused(h, w, bias, scaling):
-    """reference moe.rs route() -> rs_router_fused -> glm53_router_fused_cuda: h f32 [rows, k], w f32|bf16 [E, k]."""
+def glm_router_fused(h, w, bias, scaling, half_w=False):
+    """reference moe.rs route() -> rs_router_fused(_h) -> glm53_router_fused(_h)_cuda: h f32 [rows, k], w f32|bf16 [E, k].
+    half_w: also returns the binary16 copy of the weights that glm_moe_experts takes (reference moe.rs:66-67)."""
     rows, k = h.shape
     E = w.shape[0]
     partial = torch.empty(rows, E, 2, dtype=torch.float32, device=h.device)
     ids = torch.empty(rows, 8, dtype=torch.int64, device=h.device)
     wt = torch.empty(rows, 8, dtype=torch.float32, device=h.device)
+    if half_w:
+        wh = torch.empty(rows, 8, dtype=torch.float16, device=h.device)
+        _ck(_lib().glm53_router_fused_h_cuda(_p(_dev(h)), _p(_dev(w)), int(w.dtype == torch.bfloat16), _p(_dev(bias)), _p(partial), _p(ids), _p(wt),
+                                             _p(wh), rows, E, k, float(scaling), _st()), "glm53_router_fused_h_cuda")
+        return ids, wt, wh
     _ck(_lib().glm53_router_fused_cuda(_p(_dev(h)), _p(_dev(w)), int(w.dtype == torch.bfloat16), _p(_dev(bias)), _p(partial), _p(ids), _p(wt),
                                        rows, E, k, float(scaling), _st()), "glm53_router_fused_cuda")
     return ids, wt

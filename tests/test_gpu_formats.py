@@ -207,6 +207,11 @@ def test_glm_router_fused(ops, oracle):
     ib, wbt = ops.glm_router_fused(dev(h4), dev_bf16(wb), dev(bias), 2.5)
     lo, wo3 = oracle.glm_route((h4.astype(np.float64) @ synth.bf16_to_f32(wb).astype(np.float64).T).astype(np.float32), bias, 8, 2.5)
     assert np.array_equal(host(ib), lo) and np.allclose(host(wbt), wo3, rtol=1e-4)
+    # the form that also writes the binary16 copy of the weights (what glm_moe_experts takes): the same picks and weights, and the
+    # copy is the weights' own rounding to nearest even
+    ih, wf, wh = ops.glm_router_fused(dev(h4), dev_bf16(wb), dev(bias), 2.5, half_w=True)
+    assert np.array_equal(host(ih), host(ib)) and np.array_equal(host(wf), host(wbt))
+    assert np.array_equal(wh.cpu().numpy().view(np.uint16), host(wf).astype(np.float16).view(np.uint16))
 
 
 @pytest.mark.parametrize("m", [1, 2, 4, 7])
