@@ -230,6 +230,64 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
             const bool tail = q + NW < nkg;
             const WMat& m = t < 2 ? a.w1 : a.w3;
             const int row0 = j0 + 16 * (t & 1);
+            // Here a wave multiplies one tile with four or five K groups, so converting its activations itself would cost as many
+            // converts again as its weights do: where the rows fit, the block stages them as finished bf16 operands (thread = half a
+            // 32-block of a row, 16 values: act_quant or the caller's codes, then code x 2^scale; the two halves are lane neighbours),
+            // else as codes.  The same values either way.  The first round of pieces is requested AHEAD of the weight rows: a wave's
+            // loads return in issue order, so pieces requested behind them would arrive with the last weight row, and the barrier
+            // below would hold every wave's multiplies until the slowest wave's weights were there.
+            const bool xbf = (size_t)a.R * (2 * H + 16) <= XBF_BYTES;
+            const int xbs = 2 * H + 16;                    // row stride of the bf16 rows
+            const int nh = H >> 4, npieces = grp.n * nh;
+            struct XPiece { uint4 a, b; uint32_t sb; int r, hb; bool live; };
+            auto piece_fetch = [&](int u0) {
+                XPiece p;
+                p.live = u0 + tid < npieces;               // a round's spare threads load the last piece again and store nothing
+                const int u = p.live ? u0 + tid : npieces - 1;
+                // (the first round ahead of the weight requests without a division: more than 256 pieces a row in this branch, 512 threads)
+                p.r = u0 == 0 ? (u >= nh ? 1 : 0) : u / nh; p.hb = u - p.r * nh;
+                const int tok = rows[p.r] / a.TT;
+                if constexpr (!QUANT) {
+                    p.a = *(const uint4*)((const uint8_t*)a.x + (int64_t)tok * H + p.hb * 16);
+                    p.b = p.a;
+                    p.sb = a.xs[(int64_t)tok * (H >> 5) + (p.hb >> 1)];
+                } else {
+                    const uint4* px = (const uint4*)((const uint16_t*)a.x + (int64_t)tok * H + p.hb * 16);
+                    p.a = px[0]; p.b = px[1]; p.sb = 0u;
+                }
+                return p;
+            };
+            auto piece_put = [&](const XPiece& p) {
+                uint4 cw;
+                uint32_t sb;
+                if constexpr (!QUANT) { cw = p.a; sb = p.sb; }
+                else {
+                    const uint4 r0 = p.a, r1 = p.b;
+                    auto lo16 = [](uint32_t w) { return __uint_as_float(w << 16); };
+                    auto hi16 = [](uint32_t w) { return __uint_as_float(w & 0xffff0000u); };
+                    auto amax8 = [&](const uint4& q4) {
+                        return fmaxf(fmaxf(fmaxf(fabsf(lo16(q4.x)), fabsf(hi16(q4.x))), fmaxf(fabsf(lo16(q4.y)), fabsf(hi16(q4.y)))),
+                                     fmaxf(fmaxf(fabsf(lo16(q4.z)), fabsf(hi16(q4.z))), fmaxf(fabsf(lo16(q4.w)), fabsf(hi16(q4.w)))));
+                    };
+                    float am = fmaxf(amax8(r0), amax8(r1));
+                    am = fmaxf(am, lane_xor<1>(am, lane));
+                    sb = aq_scale(am);
+                    cw = make_uint4(aq_word4(lo16(r0.x), hi16(r0.x), lo16(r0.y), hi16(r0.y), sb), aq_word4(lo16(r0.z), hi16(r0.z), lo16(r0.w), hi16(r0.w), sb),
+                                    aq_word4(lo16(r1.x), hi16(r1.x), lo16(r1.y), hi16(r1.y), sb), aq_word4(lo16(r1.z), hi16(r1.z), lo16(r1.w), hi16(r1.w), sb));
+                }
+                const float sc = e8m0_to_f32(sb & 0xffu);
+                const uint32_t w[4] = {cw.x, cw.y, cw.z, cw.w};
+                unsigned char* d = extra + (size_t)p.r * xbs + p.hb * 32;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    bf2 v[4];
+                    v[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j], sc, false); v[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j], sc, true);
+                    v[2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j + 1], sc, false); v[3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j + 1], sc, true);
+                    uint4 w4; __builtin_memcpy(&w4, v, 16);
+                    if (p.live) *(uint4*)(d + 16 * j) = w4;
+                }
+            };
+            const XPiece first = piece_fetch(0);           // (no branch around it: valid addresses whichever way the rows are staged)
             v4i A[5][4];
             GrpScale sa[5];                                // all five requested at once; each becomes an operand when its unit is multiplied
             grp_load<LAYOUT>(m, grp.e, row0, q, lane, A[0], sa[0]);
@@ -237,50 +295,9 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
             grp_load<LAYOUT>(m, grp.e, row0, q + 2, lane, A[1], sa[1]);
             grp_load<LAYOUT>(m, grp.e, row0, q + 4, lane, A[2], sa[2]);
             grp_load<LAYOUT>(m, grp.e, row0, q + 6, lane, A[3], sa[3]);
-            // Here a wave multiplies one tile with four or five K groups, so converting its activations itself would cost as many
-            // converts again as its weights do: where the rows fit, the block stages them as finished bf16 operands (thread = one
-            // 32-block of a row: act_quant or the caller's codes, then code x 2^scale), else as codes.  The same values either way.
-            const bool xbf = (size_t)a.R * (2 * H + 16) <= XBF_BYTES;
-            const int xbs = 2 * H + 16;                    // row stride of the bf16 rows
             if (xbf) {
-                // thread = half a 32-block (16 values: few registers beside the weight rows in flight), the two halves are lane neighbours
-                const int nh = H >> 4;
-                for (int u0 = 0; u0 < grp.n * nh; u0 += NT) {
-                    const bool live = u0 + tid < grp.n * nh;                   // the last round's spare threads load the last piece again and store nothing
-                    const int u = live ? u0 + tid : grp.n * nh - 1;
-                    const int r = u / nh, hb = u - r * nh, tok = rows[r] / a.TT;
-                    uint4 cw;
-                    uint32_t sb;
-                    if constexpr (!QUANT) {
-                        cw = *(const uint4*)((const uint8_t*)a.x + (int64_t)tok * H + hb * 16);
-                        sb = a.xs[(int64_t)tok * (H >> 5) + (hb >> 1)];
-                    } else {
-                        const uint4* px = (const uint4*)((const uint16_t*)a.x + (int64_t)tok * H + hb * 16);
-                        const uint4 r0 = px[0], r1 = px[1];
-                        auto lo16 = [](uint32_t w) { return __uint_as_float(w << 16); };
-                        auto hi16 = [](uint32_t w) { return __uint_as_float(w & 0xffff0000u); };
-                        auto amax8 = [&](const uint4& q4) {
-                            return fmaxf(fmaxf(fmaxf(fabsf(lo16(q4.x)), fabsf(hi16(q4.x))), fmaxf(fabsf(lo16(q4.y)), fabsf(hi16(q4.y)))),
-                                         fmaxf(fmaxf(fabsf(lo16(q4.z)), fabsf(hi16(q4.z))), fmaxf(fabsf(lo16(q4.w)), fabsf(hi16(q4.w)))));
-                        };
-                        float am = fmaxf(amax8(r0), amax8(r1));
-                        am = fmaxf(am, lane_xor<1>(am, lane));
-                        sb = aq_scale(am);
-                        cw = make_uint4(aq_word4(lo16(r0.x), hi16(r0.x), lo16(r0.y), hi16(r0.y), sb), aq_word4(lo16(r0.z), hi16(r0.z), lo16(r0.w), hi16(r0.w), sb),
-                                        aq_word4(lo16(r1.x), hi16(r1.x), lo16(r1.y), hi16(r1.y), sb), aq_word4(lo16(r1.z), hi16(r1.z), lo16(r1.w), hi16(r1.w), sb));
-                    }
-                    const float sc = e8m0_to_f32(sb & 0xffu);
-                    const uint32_t w[4] = {cw.x, cw.y, cw.z, cw.w};
-                    unsigned char* d = extra + (size_t)r * xbs + hb * 32;
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        bf2 v[4];
-                        v[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j], sc, false); v[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j], sc, true);
-                        v[2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j + 1], sc, false); v[3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * j + 1], sc, true);
-                        uint4 w4; __builtin_memcpy(&w4, v, 16);
-                        if (live) *(uint4*)(d + 16 * j) = w4;
-                    }
-                }
+                piece_put(first);
+                for (int u0 = NT; u0 < npieces; u0 += NT) piece_put(piece_fetch(u0));
             } else stage_x(std::integral_constant<bool, !QUANT>{});
             __syncthreads();                               // a wave multiplies K groups that other waves staged
             TRACE(2);
