@@ -298,6 +298,15 @@ __global__ __launch_bounds__(NT, 4) void mx_fused_kernel(const MArgs a)
             GrpScale sa[5];                                // all five requested at once; each becomes an operand when its unit is multiplied
             grp_load<LAYOUT>(m, grp.e, row0, q, lane, A[0], sa[0]);
             if (tail) grp_load<LAYOUT>(m, grp.e, row0, q + NW, lane, A[4], sa[4]);
+            // The other three units are requested once these have arrived.  Measured, not derived (the memory system serves everything
+            // requested at once by fair share, and the exchanges queue behind all of it): all five at once 35.6 us per layer at one
+            // row of the hidden-5120 shape against 33.9 this way; the first alone and then four 34.6.
+#pragma unroll
+            for (int s = 0; s < 4; ++s) asm volatile("" : "+v"(A[0][s]));
+            if (tail) {
+#pragma unroll
+                for (int s = 0; s < 4; ++s) asm volatile("" : "+v"(A[4][s]));
+            }
             grp_load<LAYOUT>(m, grp.e, row0, q + 2, lane, A[1], sa[1]);
             grp_load<LAYOUT>(m, grp.e, row0, q + 4, lane, A[2], sa[2]);
             grp_load<LAYOUT>(m, grp.e, row0, q + 6, lane, A[3], sa[3]);
